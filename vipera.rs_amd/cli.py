@@ -217,8 +217,8 @@ def plan_model(folder: str, ctx: Optional[int], batch: int, dtype: str, block_si
             if spec.role != MATRIX or (spec.optional and not present):
                 continue
             count = 1
-            for dim in spec.shape:
-                count *= dim
+            for dim in (checkpoint.info(spec.name).shape if present else spec.shape):
+                count *= max(int(dim), 0)
             matrix_elements += count
             stored = checkpoint.info(spec.name).torch_dtype if present else run_dtype
             matrix_bytes += count * (4 if kept_dtype(spec, stored, run_dtype, keep_float32) == torch.float32 else 2)

@@ -41,6 +41,9 @@ def lookup_architecture(name: str) -> Tuple[Type[ModelConfig], Callable[..., Any
 
 
 def architecture_of(data: Dict[str, Any]) -> str:
+    """The model's class name: the first of ``architectures``, or the string under ``architecture``."""
+    if "architectures" not in data and isinstance(data.get("architecture"), str):
+        return data["architecture"]
     names = data.get("architectures")
     if not isinstance(names, list) or not names or not isinstance(names[0], str):
         raise InvalidArgumentError(

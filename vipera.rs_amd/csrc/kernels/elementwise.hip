@@ -471,3 +471,45 @@ extern "C" int vk_fill_normal(void* out, int dtype, long long count, unsigned lo
   VK_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// Dynamic Tanh: out = tanh(alpha * x) * weight + bias, elementwise (no mean, no variance); alpha is one number,
+// read from device memory.  x: 32-bit rows of `width`; rows (optional) selects them.
+template <typename TO>
+__global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, const float* __restrict__ alpha,
+                                                  const float* __restrict__ weight, const float* __restrict__ bias,
+                                                  const int* __restrict__ rows, TO* __restrict__ out, int width) {
+  const int r = blockIdx.x;
+  const float* src = x + (size_t)(rows ? rows[r] : r) * width;
+  TO* dst = out + (size_t)r * width;
+  const float a = alpha[0];
+  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = from_float<TO>(fmaf(tanhf(a * src[c]), weight[c], bias[c]));
+}
+
+extern "C" int vk_dyt(const float* x, const float* alpha, const float* weight, const float* bias, const int* rows,
+                      void* out, int out_dtype, int num_rows, int width, void* stream) {
+  if (num_rows <= 0) return 0;
+  if (width <= 0) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == DT_F32)
+    dyt_kernel<float><<<num_rows, 256, 0, s>>>(x, alpha, weight, bias, rows, (float*)out, width);
+  else if (out_dtype == DT_BF16)
+    dyt_kernel<bf16_t><<<num_rows, 256, 0, s>>>(x, alpha, weight, bias, rows, (bf16_t*)out, width);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// x *= factor, elementwise, 32-bit.
+__global__ void scale_kernel(float* __restrict__ x, float factor, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) x[i] *= factor;
+}
+
+extern "C" int vk_scale(float* x, float factor, long long count, void* stream) {
+  if (count <= 0) return 0;
+  scale_kernel<<<(unsigned)((count + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, factor, count);
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,270 @@
+// Mixture of experts: routing, grouping of (token, choice) pairs by expert, and the experts' products.
+//
+// A step's T tokens each choose `top` of E experts: P = T * top pairs, pair p = t * top + j.  The pairs are
+// grouped by expert (`order[i]` is the pair at sorted place i, `offsets[e]` the first place of expert e) and cut
+// into tiles of 64 places that never span two experts; a product's workgroup owns one tile and 64 output
+// columns.  The grid is sized for the most tiles there can be, and workgroups past `num_tiles` (which only the
+// device knows) leave at once.  Which place a pair gets depends on the order in which the counters were bumped,
+// but no value does: a pair's row is computed alone, an FMA chain in k order per output element, and the
+// weighted sum over a token's choices runs in the order of the choices.
+#include "common.h"
+
+constexpr int MOE_TILE = 64;
+
+// ---------------------------------------------------------------------------------------------
+// One wave per token: the `top` largest of E logits (the lowest id wins a tie), and the softmax over those.
+// Lane l looks after experts l, l + 64, ...; a bit per expert of its own says which are taken (E <= 4096).
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
+                                                        int num_tokens, int* __restrict__ ids,
+                                                        float* __restrict__ weights) {
+  constexpr int NONE = 0x7fffffff;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (t >= num_tokens) return;
+  const float* z = logits + (long long)t * experts;
+  unsigned long long taken = 0;
+  float first = 0.f, sum = 0.f, mine = 0.f;      // lane j keeps the weight of choice j
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int arg = NONE;
+    for (int e = lane, i = 0; e < experts; e += WAVE, ++i) {
+      if ((taken >> i) & 1ull) continue;
+      const float v = z[e];
+      if (arg == NONE || v > best) {   // ascending e: an equal later one does not replace
+        best = v;
+        arg = e;
+      }
+    }
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, WAVE);
+      const int oa = __shfl_xor(arg, off, WAVE);
+      if (oa != NONE && (arg == NONE || ob > best || (ob == best && oa < arg))) {
+        best = ob;
+        arg = oa;
+      }
+    }
+    if ((arg & (WAVE - 1)) == lane) taken |= 1ull << (arg / WAVE);
+    if (j == 0) first = best;
+    const float p = expf(best - first);
+    sum += p;
+    if (lane == j) mine = p;
+    if (lane == 0) ids[(long long)t * top + j] = arg;
+  }
+  if (lane < top) weights[(long long)t * top + lane] = mine / sum;
+}
+
+// One workgroup: counts per expert, offsets, the pairs' places, and the list of tiles.
+//   offsets [E + 1], order [P], tiles [max_tiles][2] = (expert, first place), num_tiles [1]
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int pairs, int experts,
+                                                         int* __restrict__ offsets, int* __restrict__ order,
+                                                         int* __restrict__ tiles, int* __restrict__ num_tiles) {
+  extern __shared__ int shared[];      // counts [E], cursor [E]
+  int* counts = shared;
+  int* cursor = shared + experts;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&counts[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = at;
+      cursor[e] = at;
+      for (int first = 0; first < counts[e]; first += MOE_TILE) {
+        tiles[2 * tile] = e;
+        tiles[2 * tile + 1] = at + first;
+        ++tile;
+      }
+      at += counts[e];
+    }
+    offsets[experts] = at;
+    num_tiles[0] = tile;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) order[atomicAdd(&cursor[ids[p]], 1)] = p;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gate and up products of a tile with the experts' activation:
+//   g = min(Wg h, limit), u = clamp(Wu h, -limit, limit), y = g * sigmoid(alpha * g) * (u + 1)
+// h: [T, width] (row of pair p is p / top); wg, wu: [E, ff, width]; act: [P places, ff].
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ h, long long ldh,
+                                                          const T* __restrict__ wg, const T* __restrict__ wu,
+                                                          const int* __restrict__ offsets,
+                                                          const int* __restrict__ order, const int* __restrict__ tiles,
+                                                          const int* __restrict__ num_tiles, int top, int width, int ff,
+                                                          float limit, float alpha, T* __restrict__ act) {
+  if ((int)blockIdx.x >= num_tiles[0]) return;
+  __shared__ float As[16][MOE_TILE + 4];
+  __shared__ float Gs[16][MOE_TILE + 4];
+  __shared__ float Us[16][MOE_TILE + 4];
+  __shared__ int rows[MOE_TILE];
+  const int e = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
+  const int count = min(MOE_TILE, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * MOE_TILE;
+  for (int i = threadIdx.x; i < MOE_TILE; i += 256) rows[i] = i < count ? order[first + i] / top : -1;
+  __syncthreads();
+  const T* g_w = wg + (long long)e * ff * width;
+  const T* u_w = wu + (long long)e * ff * width;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float ga[4][4] = {}, ua[4][4] = {};
+  for (int k0 = 0; k0 < width; k0 += 16) {
+    for (int i = threadIdx.x; i < MOE_TILE * 16; i += 256) {
+      const int r = i >> 4, kk = i & 15, k = k0 + kk, n = n0 + r;
+      As[kk][r] = (rows[r] >= 0 && k < width) ? to_float<T>(h[(long long)rows[r] * ldh + k]) : 0.f;
+      const bool in = n < ff && k < width;
+      Gs[kk][r] = in ? to_float<T>(g_w[(long long)n * width + k]) : 0.f;
+      Us[kk][r] = in ? to_float<T>(u_w[(long long)n * width + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float av[4], gv[4], uv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        gv[j] = Gs[kk][tx * 4 + j];
+        uv[j] = Us[kk][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          ga[i][j] = fmaf(av[i], gv[j], ga[i][j]);
+          ua[i][j] = fmaf(av[i], uv[j], ua[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r >= count) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= ff) continue;
+      const float g = fminf(ga[i][j], limit);
+      const float u = fminf(fmaxf(ua[i][j], -limit), limit);
+      const float y = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f);
+      act[(long long)(first + r) * ff + n] = from_float<T>(y);
+    }
+  }
+}
+
+// Down product of a tile: pair_out[pair, :] = Wd_e act[place, :]  (32-bit out, one row per pair).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act, const T* __restrict__ wd,
+                                                       const int* __restrict__ offsets, const int* __restrict__ order,
+                                                       const int* __restrict__ tiles, const int* __restrict__ num_tiles,
+                                                       int width, int ff, float* __restrict__ pair_out) {
+  if ((int)blockIdx.x >= num_tiles[0]) return;
+  __shared__ float As[16][MOE_TILE + 4];
+  __shared__ float Ws[16][MOE_TILE + 4];
+  const int e = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
+  const int count = min(MOE_TILE, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * MOE_TILE;
+  const T* w = wd + (long long)e * width * ff;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < ff; k0 += 16) {
+    for (int i = threadIdx.x; i < MOE_TILE * 16; i += 256) {
+      const int r = i >> 4, kk = i & 15, k = k0 + kk, n = n0 + r;
+      As[kk][r] = (r < count && k < ff) ? to_float<T>(act[(long long)(first + r) * ff + k]) : 0.f;
+      Ws[kk][r] = (n < width && k < ff) ? to_float<T>(w[(long long)n * ff + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r >= count) continue;
+    const long long pair = order[first + r];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < width) pair_out[pair * width + n] = acc[i][j];
+    }
+  }
+}
+
+// residual[t, :] += sum_j weights[t, j] * pair_out[t * top + j, :], j ascending.
+__global__ void moe_combine_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, int top,
+                                   int width, long long total, float* __restrict__ residual) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long t = idx / width;
+  const int c = (int)(idx % width);
+  float sum = 0.f;
+  for (int j = 0; j < top; ++j) sum = fmaf(weights[t * top + j], pair_out[(t * top + j) * width + c], sum);
+  residual[idx] += sum;
+}
+
+// ---------------------------------------------------------------------------------------------
+extern "C" int vk_moe_max_tiles(int pairs, int experts) { return (pairs + MOE_TILE - 1) / MOE_TILE + experts; }
+
+extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int* ids, float* weights,
+                            int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
+  if (experts > 4096) return VK_UNSUPPORTED_SIZE;
+  hipStream_t s = (hipStream_t)stream;
+  moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights);
+  VK_LAUNCH_CHECK();
+  const long long pairs = (long long)num_tokens * top;
+  if (pairs > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
+  moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(ids, (int)pairs, experts, offsets, order, tiles,
+                                                                       num_tiles);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
+                              const int* offsets, const int* order, const int* tiles, const int* num_tiles,
+                              const float* weights, int num_tokens, int experts, int top, int width, int ff,
+                              float limit, float alpha, void* act, float* pair_out, float* residual, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (experts < 1 || top < 1 || width < 1 || ff < 1) return VK_BAD_ARGUMENT;
+  const int pairs = num_tokens * top;
+  const int max_tiles = vk_moe_max_tiles(pairs, experts);
+  hipStream_t s = (hipStream_t)stream;
+  dim3 up_grid(max_tiles, (ff + MOE_TILE - 1) / MOE_TILE), down_grid(max_tiles, (width + MOE_TILE - 1) / MOE_TILE);
+  if (up_grid.y > 65535 || down_grid.y > 65535) return VK_UNSUPPORTED_SIZE;
+  if (dtype == DT_F32) {
+    moe_gate_up_kernel<float><<<up_grid, 256, 0, s>>>((const float*)h, ldh, (const float*)wg, (const float*)wu,
+                                                      offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
+                                                      (float*)act);
+    VK_LAUNCH_CHECK();
+    moe_down_kernel<float><<<down_grid, 256, 0, s>>>((const float*)act, (const float*)wd, offsets, order, tiles,
+                                                     num_tiles, width, ff, pair_out);
+  } else if (dtype == DT_BF16) {
+    moe_gate_up_kernel<bf16_t><<<up_grid, 256, 0, s>>>((const bf16_t*)h, ldh, (const bf16_t*)wg, (const bf16_t*)wu,
+                                                       offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
+                                                       (bf16_t*)act);
+    VK_LAUNCH_CHECK();
+    moe_down_kernel<bf16_t><<<down_grid, 256, 0, s>>>((const bf16_t*)act, (const bf16_t*)wd, offsets, order, tiles,
+                                                      num_tiles, width, ff, pair_out);
+  } else {
+    return VK_BAD_ARGUMENT;
+  }
+  VK_LAUNCH_CHECK();
+  const long long total = (long long)num_tokens * width;
+  moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, total, residual);
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,381 @@
+// Recurrent mixers: linear-attention layers that carry a matrix of state per head from token to token.
+//
+// Everything that enters a recurrence is 32-bit: the state, decays, gates, unit norms.  A request's state is one
+// row of a `[slots + 1, floats]` tensor; an entry that starts at position 0 treats its row as zeros, so a slot
+// that is used again needs no clearing.  The tokens of a step lie flat, entry after entry; `entry_start[e]` is
+// the first token of entry e, `entry_first_pos[e]` its position in the request, `slots[e]` the state row.
+//
+// The recurrence kernels give one lane a column of a head's state matrix (all key channels of one value
+// channel): the products with k, q and r are then sums inside a lane, in ascending key order, and do not
+// depend on what else is in the launch.  A wave owns 64 value channels of one (entry, head) and walks the
+// entry's tokens in order.
+#include "common.h"
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+// ---------------------------------------------------------------------------------------------
+// Short causal convolution over time per channel, then silu; q and k heads made unit vectors; gates.
+//   proj  [T, ldp] 32-bit: channels [q: kh*dim | k: kh*dim | v: heads*vdim] first, later columns are the caller's
+//   conv  [C, taps] 32-bit, the last column is the current token's
+//   state row: `(taps - 1) * C` floats from `conv_offset` on, the inputs of the last taps - 1 tokens, oldest first
+//   ba    columns `b_col + h` and `a_col + h` of proj hold the projections for beta and the decay's step
+// Outputs (32-bit): qkv [T, C] (q unit * dim^-1/2, k unit, v), beta [T, heads], decay [T, heads].
+// One workgroup per token.
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    const float* __restrict__ proj, long long ldp, const float* __restrict__ conv, int taps,
+    const float* __restrict__ state, long long state_stride, long long conv_offset, const int* __restrict__ entry_of,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias, int kv_heads, int dim, int heads, int vdim,
+    int b_col, int a_col, float unit_eps, float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
+  extern __shared__ float row[];   // C floats
+  const int t = blockIdx.x;
+  const int e = entry_of[t];
+  const int start = entry_start[e];
+  const int offset = t - start;
+  const bool fresh = entry_first[e] == 0;
+  const int C = 2 * kv_heads * dim + heads * vdim;
+  const float* old = state + (long long)slots[e] * state_stride + conv_offset;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float sum = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;            // how many tokens before this one
+      float x;
+      if (back <= offset) {
+        x = proj[(long long)(t - back) * ldp + c];
+      } else if (fresh) {
+        x = 0.f;
+      } else {
+        x = old[(long long)(taps - 1 - (back - offset)) * C + c];   // back - offset tokens before the entry
+      }
+      sum = fmaf(conv[(long long)c * taps + j], x, sum);
+    }
+    row[c] = silu_f(sum);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+  float* out = qkv + (long long)t * C;
+  const int unit_heads = 2 * kv_heads;
+  for (int h = wave; h < unit_heads; h += waves) {
+    const float* src = row + h * dim;
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += WAVE) ss += src[d] * src[d];
+    ss = wave_sum(ss);
+    float inv = 1.0f / sqrtf(ss + unit_eps);
+    if (h < kv_heads) inv *= 1.0f / sqrtf((float)dim);
+    for (int d = lane; d < dim; d += WAVE) out[h * dim + d] = src[d] * inv;
+  }
+  for (int c = unit_heads * dim + threadIdx.x; c < C; c += blockDim.x) out[c] = row[c];
+  for (int h = threadIdx.x; h < heads; h += blockDim.x) {
+    const float* p = proj + (long long)t * ldp;
+    beta[(long long)t * heads + h] = sigmoid_f(p[b_col + h]);
+    decay[(long long)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(p[a_col + h] + dt_bias[h]));
+  }
+}
+
+// The convolution's inputs of an entry's last taps - 1 tokens become the state.  One workgroup per entry; runs
+// after delta_prepare has read the old rows.
+__global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict__ proj, long long ldp, int taps, int C,
+                                                         float* __restrict__ state, long long state_stride,
+                                                         long long conv_offset, const int* __restrict__ entry_start,
+                                                         const int* __restrict__ entry_first,
+                                                         const int* __restrict__ slots) {
+  const int e = blockIdx.x;
+  const int start = entry_start[e], count = entry_start[e + 1] - start;
+  const bool fresh = entry_first[e] == 0;
+  float* rows = state + (long long)slots[e] * state_stride + conv_offset;
+  const int keep = taps - 1;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    for (int j = 0; j < keep; ++j) {           // ascending: row j + count is read before it is written
+      const int from = j + count;              // index into [old rows (keep) | the entry's tokens (count)]
+      float x;
+      if (from >= keep) x = proj[(long long)(start + from - keep) * ldp + c];
+      else x = fresh ? 0.f : rows[(long long)from * C + c];
+      rows[(long long)j * C + c] = x;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gated delta rule.  Per head, with S [dim, vdim]:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
+// Grid (entries, heads, ceil(vdim / 64)), one wave each.  Dynamic LDS: dim * 64 floats of state and 2 * dim of k, q.
+__global__ __launch_bounds__(64) void delta_rule_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
+    float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
+    const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
+    float* __restrict__ out) {
+  extern __shared__ float lds[];
+  float* S = lds;                    // [dim][64]
+  float* ks = lds + dim * WAVE;      // [dim]
+  float* qs = ks + dim;              // [dim]
+  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int v = blockIdx.z * WAVE + lane;
+  const bool live = v < vdim;
+  const int kh = h / (heads / kv_heads);
+  const int C = 2 * kv_heads * dim + heads * vdim;
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * vdim;
+  const bool fresh = entry_first[e] == 0;
+  for (int d = 0; d < dim; ++d) S[d * WAVE + lane] = (live && !fresh) ? mine[(long long)d * vdim + v] : 0.f;
+  for (int t = start; t < end; ++t) {
+    const float* row = qkv + (long long)t * C;
+    __syncthreads();
+    for (int d = lane; d < dim; d += WAVE) {
+      qs[d] = row[kh * dim + d];
+      ks[d] = row[(kv_heads + kh) * dim + d];
+    }
+    __syncthreads();
+    const float g = decay[(long long)t * heads + h], b = beta[(long long)t * heads + h];
+    const float val = live ? row[2 * kv_heads * dim + h * vdim + v] : 0.f;
+    float dot = 0.f;
+    for (int d = 0; d < dim; ++d) {
+      const float s = g * S[d * WAVE + lane];
+      S[d * WAVE + lane] = s;
+      dot = fmaf(s, ks[d], dot);
+    }
+    const float u = b * (val - dot);
+    float o = 0.f;
+    for (int d = 0; d < dim; ++d) {
+      const float s = fmaf(ks[d], u, S[d * WAVE + lane]);
+      S[d * WAVE + lane] = s;
+      o = fmaf(s, qs[d], o);
+    }
+    if (live) out[((long long)t * heads + h) * vdim + v] = o;
+  }
+  if (live)
+    for (int d = 0; d < dim; ++d) mine[(long long)d * vdim + v] = S[d * WAVE + lane];
+}
+
+// ---------------------------------------------------------------------------------------------
+// RWKV-style time mixing.  Per head, with S [dim, dim]:  o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T,
+// w = exp(-exp(wraw + w0)) per key channel.  r, k, v, wraw are 32-bit [T, heads * dim] with row strides of their own.
+// Grid (entries, heads, ceil(dim / 64)), one wave each.  Dynamic LDS: dim * 64 floats of state and 3 * dim floats.
+__global__ __launch_bounds__(64) void wkv_rule_kernel(
+    const float* __restrict__ r, long long ldr, const float* __restrict__ k, long long ldk, const float* __restrict__ v,
+    long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
+    const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
+    int heads, float* __restrict__ out) {
+  extern __shared__ float lds[];
+  float* S = lds;                    // [dim][64]
+  float* rs = lds + dim * WAVE;      // r[d]
+  float* ks = rs + dim;              // k[d]
+  float* ws = ks + dim;              // decay[d]
+  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int col = blockIdx.z * WAVE + lane;
+  const bool live = col < dim;
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * dim;
+  const bool fresh = entry_first[e] == 0;
+  for (int d = 0; d < dim; ++d) S[d * WAVE + lane] = (live && !fresh) ? mine[(long long)d * dim + col] : 0.f;
+  for (int t = start; t < end; ++t) {
+    __syncthreads();
+    for (int d = lane; d < dim; d += WAVE) {
+      rs[d] = r[(long long)t * ldr + h * dim + d];
+      ks[d] = k[(long long)t * ldk + h * dim + d];
+      ws[d] = expf(-expf(wraw[(long long)t * ldw + h * dim + d] + w0[h * dim + d]));
+    }
+    __syncthreads();
+    const float val = live ? v[(long long)t * ldv + h * dim + col] : 0.f;
+    float o = 0.f;
+    for (int d = 0; d < dim; ++d) {
+      const float kv = ks[d] * val;
+      const float s = S[d * WAVE + lane];
+      o = fmaf(fmaf(bonus[h * dim + d], kv, s), rs[d], o);
+      S[d * WAVE + lane] = fmaf(ws[d], s, kv);
+    }
+    if (live) out[((long long)t * heads + h) * dim + col] = o;
+  }
+  if (live)
+    for (int d = 0; d < dim; ++d) mine[(long long)d * dim + col] = S[d * WAVE + lane];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Token shift: mix_s[t] = h[t] + (h[t-1] - h[t]) * mu_s for `mixes` vectors mu; h[t-1] of an entry's first token
+// is the state's saved row (zeros at position 0).  out [mixes, T, width] in the run's dtype.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ h, int width, const float* __restrict__ mu,
+                                                          int mixes, const float* __restrict__ state,
+                                                          long long state_stride, long long prev_offset,
+                                                          const int* __restrict__ entry_of,
+                                                          const int* __restrict__ entry_start,
+                                                          const int* __restrict__ entry_first,
+                                                          const int* __restrict__ slots, int num_tokens,
+                                                          T* __restrict__ out) {
+  const int t = blockIdx.x;
+  const int e = entry_of[t];
+  const bool first = t == entry_start[e];
+  const bool fresh = entry_first[e] == 0;
+  const float* saved = state + (long long)slots[e] * state_stride + prev_offset;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float cur = to_float<T>(h[(long long)t * width + c]);
+    const float prev = first ? (fresh ? 0.f : saved[c]) : to_float<T>(h[(long long)(t - 1) * width + c]);
+    const float diff = prev - cur;
+    for (int s = 0; s < mixes; ++s)
+      out[((long long)s * num_tokens + t) * width + c] = from_float<T>(fmaf(diff, mu[(long long)s * width + c], cur));
+  }
+}
+
+// An entry's last h becomes the state's saved row; one workgroup per entry, after token_shift has read the old one.
+template <typename T>
+__global__ __launch_bounds__(256) void save_last_kernel(const T* __restrict__ h, int width, float* __restrict__ state,
+                                                        long long state_stride, long long prev_offset,
+                                                        const int* __restrict__ entry_start,
+                                                        const int* __restrict__ slots) {
+  const int e = blockIdx.x;
+  const int last = entry_start[e + 1] - 1;
+  float* saved = state + (long long)slots[e] * state_stride + prev_offset;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) saved[c] = to_float<T>(h[(long long)last * width + c]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Read-out of a recurrent head: o / rms(o) (per head, over its `vdim` channels) * weight * gate.
+// weight: [vdim] shared by the heads, or [heads * vdim]; gate: a column range of a [T, ldg] buffer of type TG,
+// passed through silu first if asked.  One wave per (token, head).
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ weight,
+                                                             int weight_per_head, const TG* __restrict__ gate,
+                                                             long long ldg, int gate_silu, float eps, int heads,
+                                                             int vdim, int num_tokens, TO* __restrict__ out) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const long long unit = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (unit >= (long long)num_tokens * heads) return;
+  const int t = (int)(unit / heads), h = (int)(unit % heads);
+  const float* src = o + unit * vdim;
+  float ss = 0.f;
+  for (int c = lane; c < vdim; c += WAVE) ss += src[c] * src[c];
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  for (int c = lane; c < vdim; c += WAVE) {
+    float g = to_float<TG>(gate[(long long)t * ldg + h * vdim + c]);
+    if (gate_silu) g = silu_f(g);
+    const float w = weight[(weight_per_head ? h * vdim : 0) + c];
+    out[unit * vdim + c] = from_float<TO>(src[c] * inv * w * g);
+  }
+}
+
+// out = tanh(x), elementwise, 32-bit in, TO out.
+template <typename TO>
+__global__ void tanh_kernel(const float* __restrict__ x, TO* __restrict__ out, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) out[i] = from_float<TO>(tanhf(x[i]));
+}
+
+// ---------------------------------------------------------------------------------------------
+static inline bool fits_lds(long long bytes) { return bytes <= 64 * 1024; }
+
+extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* conv, int taps, float* state,
+                                long long state_stride, long long conv_offset, const int* entry_of,
+                                const int* entry_start, const int* entry_first, const int* slots, const float* a_log,
+                                const float* dt_bias, int kv_heads, int dim, int heads, int vdim, int b_col, int a_col,
+                                float unit_eps, float* qkv, float* beta, float* decay, int num_tokens, int num_entries,
+                                void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (taps < 1 || kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
+  const long long C = 2LL * kv_heads * dim + (long long)heads * vdim;
+  if (!fits_lds(C * 4)) return VK_UNSUPPORTED_SIZE;
+  hipStream_t s = (hipStream_t)stream;
+  delta_prepare_kernel<<<num_tokens, 256, (size_t)C * 4, s>>>(proj, ldp, conv, taps, state, state_stride, conv_offset,
+                                                              entry_of, entry_start, entry_first, slots, a_log, dt_bias,
+                                                              kv_heads, dim, heads, vdim, b_col, a_col, unit_eps, qkv,
+                                                              beta, decay);
+  VK_LAUNCH_CHECK();
+  if (taps > 1) {
+    conv_state_kernel<<<num_entries, 256, 0, s>>>(proj, ldp, taps, (int)C, state, state_stride, conv_offset,
+                                                  entry_start, entry_first, slots);
+    VK_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
+                             long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
+                             int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, void* stream) {
+  if (num_entries <= 0) return 0;
+  if (kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
+  const long long bytes = ((long long)dim * WAVE + 2LL * dim) * 4;
+  if (!fits_lds(bytes) || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  dim3 grid(num_entries, heads, (vdim + WAVE - 1) / WAVE);
+  delta_rule_kernel<<<grid, WAVE, (size_t)bytes, (hipStream_t)stream>>>(qkv, beta, decay, state, state_stride,
+                                                                        entry_start, entry_first, slots, kv_heads, dim,
+                                                                        heads, vdim, out);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv,
+                           const float* wraw, long long ldw, const float* w0, const float* bonus, float* state,
+                           long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
+                           int dim, int heads, float* out, int num_entries, void* stream) {
+  if (num_entries <= 0) return 0;
+  if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
+  const long long bytes = ((long long)dim * WAVE + 3LL * dim) * 4;
+  if (!fits_lds(bytes) || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  dim3 grid(num_entries, heads, (dim + WAVE - 1) / WAVE);
+  wkv_rule_kernel<<<grid, WAVE, (size_t)bytes, (hipStream_t)stream>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus,
+                                                                      state, state_stride, entry_start, entry_first,
+                                                                      slots, dim, heads, out);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_token_shift(const void* h, int dtype, int width, const float* mu, int mixes, float* state,
+                              long long state_stride, long long prev_offset, const int* entry_of,
+                              const int* entry_start, const int* entry_first, const int* slots, int num_tokens,
+                              int num_entries, void* out, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (width < 1 || mixes < 1) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32) {
+    token_shift_kernel<float><<<num_tokens, 256, 0, s>>>((const float*)h, width, mu, mixes, state, state_stride,
+                                                         prev_offset, entry_of, entry_start, entry_first, slots,
+                                                         num_tokens, (float*)out);
+    VK_LAUNCH_CHECK();
+    save_last_kernel<float><<<num_entries, 256, 0, s>>>((const float*)h, width, state, state_stride, prev_offset,
+                                                        entry_start, slots);
+  } else if (dtype == DT_BF16) {
+    token_shift_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((const bf16_t*)h, width, mu, mixes, state, state_stride,
+                                                          prev_offset, entry_of, entry_start, entry_first, slots,
+                                                          num_tokens, (bf16_t*)out);
+    VK_LAUNCH_CHECK();
+    save_last_kernel<bf16_t><<<num_entries, 256, 0, s>>>((const bf16_t*)h, width, state, state_stride, prev_offset,
+                                                         entry_start, slots);
+  } else {
+    return VK_BAD_ARGUMENT;
+  }
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_head_norm_gate(const float* o, const float* weight, int weight_per_head, const void* gate,
+                                 int gate_dtype, long long ldg, int gate_silu, float eps, int heads, int vdim,
+                                 int num_tokens, void* out, int out_dtype, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads < 1 || vdim < 1) return VK_BAD_ARGUMENT;
+  const long long units = (long long)num_tokens * heads;
+  const unsigned blocks = (unsigned)((units + 3) / 4);
+  hipStream_t s = (hipStream_t)stream;
+#define VK_HNG(TG, TO)                                                                                         \
+  head_norm_gate_kernel<TG, TO><<<blocks, 256, 0, s>>>(o, weight, weight_per_head, (const TG*)gate, ldg,      \
+                                                       gate_silu, eps, heads, vdim, num_tokens, (TO*)out)
+  if (gate_dtype == DT_F32 && out_dtype == DT_F32) VK_HNG(float, float);
+  else if (gate_dtype == DT_F32 && out_dtype == DT_BF16) VK_HNG(float, bf16_t);
+  else if (gate_dtype == DT_BF16 && out_dtype == DT_BF16) VK_HNG(bf16_t, bf16_t);
+  else if (gate_dtype == DT_BF16 && out_dtype == DT_F32) VK_HNG(bf16_t, float);
+  else return VK_BAD_ARGUMENT;
+#undef VK_HNG
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_tanh(const float* x, void* out, int out_dtype, long long count, void* stream) {
+  if (count <= 0) return 0;
+  const unsigned blocks = (unsigned)((count + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == DT_F32) tanh_kernel<float><<<blocks, 256, 0, s>>>(x, (float*)out, count);
+  else if (out_dtype == DT_BF16) tanh_kernel<bf16_t><<<blocks, 256, 0, s>>>(x, (bf16_t*)out, count);
+  else return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -35,6 +35,9 @@ MODULES: Dict[str, tuple] = {
     "attn_generic": ("hip", ["kernels/attn_generic.hip"], ["kernels/common.h"]),
     "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h", "kernels/no_alloc.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
+    "recurrent": ("hip", ["kernels/recurrent.hip"], ["kernels/common.h"]),
+    "latent": ("hip", ["kernels/latent.hip"], ["kernels/common.h"]),
+    "moe": ("hip", ["kernels/moe.hip"], ["kernels/common.h"]),
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
              ["host/cache_manager.h", "host/scheduler.h"]),
 }

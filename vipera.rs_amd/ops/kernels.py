@@ -876,3 +876,286 @@ def gemm_bf16_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows_pe
     ldc = out.stride(0) if m > 1 else max(out.stride(0), n // 2)
     fn = _fn("gemm_bf16", "vk_gemm_bf16_gated", [_p, _p, _p, _i, _i, _i, _ll, _ll, _i, _p])
     _status(fn(_ptr(a), _ptr(w), _ptr(out), m, n, k, lda, ldc, int(rows_per_wave), _stream()), "gemm_bf16_gated")
+
+
+# ----------------------------------------------------------------------------------------------
+def _f32(tensor: torch.Tensor, what: str) -> None:
+    _need(tensor.dtype == torch.float32 and tensor.is_contiguous(), f"{what} must be contiguous float32")
+
+
+def _i32(*tensors: torch.Tensor) -> None:
+    for tensor in tensors:
+        _need(tensor.dtype == torch.int32 and tensor.is_contiguous(), "index tensors must be contiguous int32")
+
+
+def dyt(x: torch.Tensor, alpha: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, out: torch.Tensor,
+        rows: Optional[torch.Tensor] = None) -> None:
+    """``out = tanh(alpha * x) * weight + bias`` per element; ``x`` 32-bit ``[tokens, width]``, ``alpha`` one number
+    on the device; ``rows`` (int32) selects rows of ``x``."""
+    _dev(x, alpha, weight, bias, out, rows)
+    width = x.shape[1]
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "dyt: x must be contiguous float32 [tokens, width]")
+    _need(alpha.dtype == torch.float32 and alpha.numel() == 1, "dyt: alpha must be one float32")
+    for name, t in (("weight", weight), ("bias", bias)):
+        _need(t.dtype == torch.float32 and t.numel() == width and t.is_contiguous(), f"dyt: {name} must be float32 [width]")
+    count = x.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows)
+    _need(out.shape == (count, width) and out.is_contiguous(), "dyt: out shape")
+    fn = _fn("elementwise", "vk_dyt", [_p, _p, _p, _p, _p, _p, _i, _i, _i, _p])
+    _status(fn(_ptr(x), _ptr(alpha), _ptr(weight), _ptr(bias), _ptr(rows), _ptr(out), _dt(out, "out"), count, width,
+               _stream()), "dyt")
+
+
+def scale_(x: torch.Tensor, factor: float) -> None:
+    """``x *= factor`` (32-bit, in place)."""
+    _dev(x)
+    _f32(x, "scale: x")
+    fn = _fn("elementwise", "vk_scale", [_p, _f, _ll, _p])
+    _status(fn(_ptr(x), float(factor), x.numel(), _stream()), "scale")
+
+
+def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = tanh(x)``; ``x`` 32-bit, ``out`` of either dtype."""
+    _dev(x, out)
+    _f32(x, "tanh: x")
+    _need(out.numel() == x.numel() and out.is_contiguous(), "tanh: out")
+    fn = _fn("recurrent", "vk_tanh", [_p, _p, _i, _ll, _p])
+    _status(fn(_ptr(x), _ptr(out), _dt(out, "out"), x.numel(), _stream()), "tanh")
+
+
+# --- recurrent mixers ---------------------------------------------------------------------------
+RECURRENT_MAX_KEY_DIM = 240    # a wave's 64 columns of a head's state and its k, q (r, decay) rows share 64 KB of LDS
+
+
+def _entries_ok(batch_arrays, num_entries: int) -> None:
+    entry_start, entry_first, slots = batch_arrays
+    _i32(entry_start, entry_first, slots)
+    _need(entry_start.numel() >= num_entries + 1 and entry_first.numel() >= num_entries and slots.numel() >= num_entries,
+          "recurrent: entry arrays are shorter than the number of entries")
+
+
+def delta_prepare(proj: torch.Tensor, conv: torch.Tensor, state: torch.Tensor, conv_offset: int, entry_of: torch.Tensor,
+                  entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, a_log: torch.Tensor,
+                  dt_bias: torch.Tensor, kv_heads: int, dim: int, heads: int, vdim: int, b_col: int, a_col: int,
+                  unit_eps: float, qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, num_entries: int) -> None:
+    """Short causal convolution, silu, unit norms of q and k, beta and the decay for every token of the step (see
+    ``recurrent.hip``); then the convolution's state rows are replaced by the entries' last inputs."""
+    _dev(proj, conv, state, entry_of, entry_start, entry_first, slots, a_log, dt_bias, qkv, beta, decay)
+    tokens = proj.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    taps = conv.shape[1]
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "delta_prepare: proj")
+    _need(proj.shape[1] >= max(channels, b_col + heads, a_col + heads) and min(b_col, a_col) >= 0, "delta_prepare: columns")
+    _need(conv.shape == (channels, taps) and taps >= 1, "delta_prepare: conv shape")
+    _f32(conv, "delta_prepare: conv")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and conv_offset + (taps - 1) * channels <= state.shape[1], "delta_prepare: state row")
+    _i32(entry_of)
+    _need(entry_of.numel() >= tokens, "delta_prepare: entry_of")
+    _entries_ok((entry_start, entry_first, slots), num_entries)
+    for name, t in (("a_log", a_log), ("dt_bias", dt_bias)):
+        _need(t.dtype == torch.float32 and t.numel() == heads, f"delta_prepare: {name}")
+    _need(qkv.shape == (tokens, channels) and beta.shape == (tokens, heads) and decay.shape == (tokens, heads),
+          "delta_prepare: output shapes")
+    for t in (qkv, beta, decay):
+        _f32(t, "delta_prepare: outputs")
+    fn = _fn("recurrent", "vk_delta_prepare",
+             [_p, _ll, _p, _i, _p, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _p, _p, _p, _i, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), _ptr(conv), taps, _ptr(state), state.stride(0), conv_offset, _ptr(entry_of),
+               _ptr(entry_start), _ptr(entry_first), _ptr(slots), _ptr(a_log), _ptr(dt_bias), kv_heads, dim, heads, vdim,
+               b_col, a_col, float(unit_eps), _ptr(qkv), _ptr(beta), _ptr(decay), tokens, num_entries, _stream()),
+            "delta_prepare")
+
+
+def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+               entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, kv_heads: int, dim: int,
+               heads: int, vdim: int, out: torch.Tensor, num_entries: int) -> None:
+    """The gated delta rule over every entry's tokens in order, from and into the entries' state rows (the first
+    ``heads * dim * vdim`` floats of a row, ``[heads, dim, vdim]``); ``out`` 32-bit ``[tokens, heads * vdim]``."""
+    _dev(qkv, beta, decay, state, entry_start, entry_first, slots, out)
+    tokens = qkv.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    _need(qkv.shape == (tokens, channels) and beta.shape == (tokens, heads) and decay.shape == (tokens, heads)
+          and out.shape == (tokens, heads * vdim), "delta_rule: shapes")
+    for t in (qkv, beta, decay, out):
+        _f32(t, "delta_rule: operands")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= heads * dim * vdim, "delta_rule: state row")
+    _entries_ok((entry_start, entry_first, slots), num_entries)
+    if dim > RECURRENT_MAX_KEY_DIM:
+        raise UnsupportedError(f"delta_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
+    fn = _fn("recurrent", "vk_delta_rule", [_p, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(qkv), _ptr(beta), _ptr(decay), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first),
+               _ptr(slots), kv_heads, dim, heads, vdim, _ptr(out), num_entries, _stream()), "delta_rule")
+
+
+def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor,
+             bonus: torch.Tensor, state: torch.Tensor, entry_start: torch.Tensor, entry_first: torch.Tensor,
+             slots: torch.Tensor, dim: int, heads: int, out: torch.Tensor, num_entries: int) -> None:
+    """RWKV-style time mixing over every entry's tokens in order: ``o = (S + diag(u) k v^T)^T r``, then
+    ``S = diag(w) S + k v^T`` with ``w = exp(-exp(wraw + w0))``.  ``r, k, v, wraw``: 32-bit ``[tokens, heads * dim]``
+    (row-strided views are fine); state rows start with ``[heads, dim, dim]``."""
+    _dev(r, k, v, wraw, w0, bonus, state, entry_start, entry_first, slots, out)
+    tokens, width = out.shape[0], heads * dim
+    for name, t in (("r", r), ("k", k), ("v", v), ("wraw", wraw)):
+        _need(t.dtype == torch.float32 and t.shape == (tokens, width) and t.stride(1) == 1, f"wkv_rule: {name}")
+    for name, t in (("w0", w0), ("bonus", bonus)):
+        _need(t.dtype == torch.float32 and t.numel() == width and t.is_contiguous(), f"wkv_rule: {name}")
+    _f32(out, "wkv_rule: out")
+    _need(out.shape == (tokens, width), "wkv_rule: out shape")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= heads * dim * dim, "wkv_rule: state row")
+    _entries_ok((entry_start, entry_first, slots), num_entries)
+    if dim > RECURRENT_MAX_KEY_DIM:
+        raise UnsupportedError(f"wkv_rule: a head width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
+    fn = _fn("recurrent", "vk_wkv_rule",
+             [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(wraw), wraw.stride(0), _ptr(w0),
+               _ptr(bonus), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first), _ptr(slots), dim, heads,
+               _ptr(out), num_entries, _stream()), "wkv_rule")
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_offset: int, entry_of: torch.Tensor,
+                entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, out: torch.Tensor,
+                num_entries: int) -> None:
+    """``out[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s]``; the token before an entry's first is the state's saved row
+    (``width`` floats from ``prev_offset`` on; zeros at position 0), which then takes the entry's last ``h``."""
+    _dev(h, mu, state, entry_of, entry_start, entry_first, slots, out)
+    tokens, width = h.shape
+    mixes = mu.shape[0]
+    _need(h.is_contiguous() and out.dtype == h.dtype and out.shape == (mixes, tokens, width) and out.is_contiguous(),
+          "token_shift: h and out")
+    _need(mu.dtype == torch.float32 and mu.shape == (mixes, width) and mu.is_contiguous(), "token_shift: mu")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and prev_offset + width <= state.shape[1], "token_shift: state row")
+    _i32(entry_of)
+    _need(entry_of.numel() >= tokens, "token_shift: entry_of")
+    _entries_ok((entry_start, entry_first, slots), num_entries)
+    fn = _fn("recurrent", "vk_token_shift", [_p, _i, _i, _p, _i, _p, _ll, _ll, _p, _p, _p, _p, _i, _i, _p, _p])
+    _status(fn(_ptr(h), _dt(h, "h"), width, _ptr(mu), mixes, _ptr(state), state.stride(0), prev_offset, _ptr(entry_of),
+               _ptr(entry_start), _ptr(entry_first), _ptr(slots), tokens, num_entries, _ptr(out), _stream()), "token_shift")
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_silu: bool, eps: float, heads: int,
+                   vdim: int, out: torch.Tensor) -> None:
+    """``out[t, h] = o[t, h] / rms(o[t, h]) * weight * gate[t, h]`` per head of ``vdim`` channels; ``weight`` is
+    ``[vdim]`` (shared by the heads) or ``[heads * vdim]``; ``gate`` (a row-strided view of either dtype) goes through
+    silu first if ``gate_silu``."""
+    _dev(o, weight, gate, out)
+    tokens = o.shape[0]
+    _f32(o, "head_norm_gate: o")
+    _need(o.shape == (tokens, heads * vdim) and out.shape == o.shape and out.is_contiguous(), "head_norm_gate: shapes")
+    _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() in (vdim, heads * vdim),
+          "head_norm_gate: weight")
+    _need(gate.shape == o.shape and gate.stride(1) == 1, "head_norm_gate: gate")
+    fn = _fn("recurrent", "vk_head_norm_gate", [_p, _p, _i, _p, _i, _ll, _i, _f, _i, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(o), _ptr(weight), 1 if weight.numel() == heads * vdim and heads > 1 else 0, _ptr(gate),
+               _dt(gate, "gate"), gate.stride(0), 1 if gate_silu else 0, float(eps), heads, vdim, tokens, _ptr(out),
+               _dt(out, "out"), _stream()), "head_norm_gate")
+
+
+# --- latent attention -----------------------------------------------------------------------------
+def latent_kv_write(x: torch.Tensor, weight: torch.Tensor, eps: float, rank: int, rot: int, rot_dims: int,
+                    positions: torch.Tensor, inv_freq: Optional[torch.Tensor], entry_of: torch.Tensor,
+                    table: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """A step's cached rows ``[rms_norm(x[:rank]) * weight | rotate(x[rank:rank + rot])]`` into their pages, as keys
+    and transposed as values (one key head of width ``rank + rot``).  ``x``: a 32-bit row-strided view."""
+    _dev(x, weight, positions, inv_freq, entry_of, table, k_cache, v_cache)
+    tokens = x.shape[0]
+    width = rank + rot
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1 and x.shape[1] == width, "latent_kv_write: x")
+    _need(weight.dtype == torch.float32 and weight.numel() == rank and weight.is_contiguous(), "latent_kv_write: weight")
+    _need(_cache_ok(k_cache, v_cache, 1, width, k_cache.dtype), "latent_kv_write: cache shape")
+    _i32(positions, entry_of, table)
+    _need(positions.numel() >= tokens and entry_of.numel() >= tokens and table.dim() == 2, "latent_kv_write: indices")
+    _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2),
+          "latent_kv_write: inv_freq")
+    fn = _fn("latent", "vk_latent_kv_write", [_p, _ll, _p, _f, _i, _i, _i, _p, _p, _p, _p, _i, _i, _p, _p, _i, _i, _p])
+    _status(fn(_ptr(x), x.stride(0), _ptr(weight), float(eps), rank, rot, rot_dims, _ptr(positions), _ptr(inv_freq),
+               _ptr(entry_of), _ptr(table), table.shape[1], k_cache.shape[2], _ptr(k_cache), _ptr(v_cache),
+               _dt(k_cache, "cache"), tokens, _stream()), "latent_kv_write")
+
+
+def latent_q_rotate(q: torch.Tensor, q_head: int, q_offset: int, out: torch.Tensor, out_head: int, out_offset: int,
+                    heads: int, rot: int, rot_dims: int, positions: torch.Tensor, inv_freq: Optional[torch.Tensor]) -> None:
+    """``out[t, h, out_offset:out_offset + rot] = rotate(q[t, h, q_offset:q_offset + rot])`` for every head."""
+    _dev(q, out, positions, inv_freq)
+    tokens = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * q_head and q_offset + rot <= q_head, "latent_q_rotate: q")
+    _need(out.dtype == q.dtype and out.is_contiguous() and out.shape == (tokens, heads * out_head)
+          and out_offset + rot <= out_head, "latent_q_rotate: out")
+    _i32(positions)
+    _need(rot_dims == 0 or (inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2),
+          "latent_q_rotate: inv_freq")
+    fn = _fn("latent", "vk_latent_q_rotate", [_p, _ll, _i, _i, _p, _i, _i, _i, _i, _i, _p, _p, _i, _i, _p])
+    _status(fn(_ptr(q), q.stride(0), q_head, q_offset, _ptr(out), out_head, out_offset, heads, rot, rot_dims,
+               _ptr(positions), _ptr(inv_freq), _dt(q, "q"), tokens, _stream()), "latent_q_rotate")
+
+
+def head_linear(a: torch.Tensor, a_head_stride: int, k: int, w: torch.Tensor, out: torch.Tensor,
+                out_head_stride: int) -> None:
+    """A product per head: ``out[t, h*so : h*so + N] = w[h] @ a[t, h*sa : h*sa + K]``; ``w``: ``[heads, N, K]``."""
+    _dev(a, w, out)
+    heads, n, kw = w.shape
+    tokens = a.shape[0]
+    _need(kw == k and w.is_contiguous(), "head_linear: w")
+    _need(a.dim() == 2 and a.stride(1) == 1 and (heads - 1) * a_head_stride + k <= a.shape[1], "head_linear: a")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[0] == tokens
+          and (heads - 1) * out_head_stride + n <= out.shape[1], "head_linear: out")
+    fn = _fn("latent", "vk_head_linear", [_p, _i, _ll, _ll, _p, _i, _p, _i, _ll, _ll, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(a), _dt(a, "a"), a.stride(0), a_head_stride, _ptr(w), _dt(w, "w"), _ptr(out), _dt(out, "out"),
+               out.stride(0), out_head_stride, tokens, n, k, heads, _stream()), "head_linear")
+
+
+# --- mixture of experts ---------------------------------------------------------------------------
+MOE_TILE = 64
+
+
+def moe_max_tiles(pairs: int, experts: int) -> int:
+    return (pairs + MOE_TILE - 1) // MOE_TILE + experts
+
+
+def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, offsets: torch.Tensor,
+              order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor) -> None:
+    """Each token's ``top`` largest router logits (lowest id first among equals) with the softmax over those, and the
+    (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``."""
+    _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
+    tokens, experts = logits.shape
+    _f32(logits, "moe_route: logits")
+    _need(1 <= top <= min(experts, 64), f"moe_route: top {top} of {experts} experts")
+    _i32(ids, offsets, order, tiles, num_tiles)
+    _f32(weights, "moe_route: weights")
+    _need(ids.numel() == tokens * top and weights.numel() == tokens * top and order.numel() == tokens * top
+          and offsets.numel() == experts + 1 and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts)
+          and num_tiles.numel() == 1, "moe_route: output sizes")
+    fn = _fn("moe", "vk_moe_route", [_p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
+    _status(fn(_ptr(logits), experts, top, tokens, _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles),
+               _ptr(num_tiles), _stream()), "moe_route")
+
+
+def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
+                order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, weights: torch.Tensor, top: int,
+                limit: float, alpha: float, act: torch.Tensor, pair_out: torch.Tensor, residual: torch.Tensor) -> None:
+    """The chosen experts of every token: ``y = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(Wg h, limit)`` and
+    ``u = clamp(Wu h, -limit, limit)``, then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])``."""
+    _dev(h, w_gate, w_up, w_down, offsets, order, tiles, num_tiles, weights, act, pair_out, residual)
+    tokens, width = h.shape
+    experts, ff, _ = w_gate.shape
+    _need(h.stride(1) == 1 and w_gate.shape == (experts, ff, width) and w_up.shape == w_gate.shape
+          and w_down.shape == (experts, width, ff), "moe_experts: weight shapes")
+    for t in (w_gate, w_up, w_down):
+        _need(t.dtype == h.dtype and t.is_contiguous(), "moe_experts: weights must be contiguous and of h's dtype")
+    _need(act.dtype == h.dtype and act.shape == (tokens * top, ff) and act.is_contiguous(), "moe_experts: act")
+    _f32(pair_out, "moe_experts: pair_out")
+    _f32(residual, "moe_experts: residual")
+    _f32(weights, "moe_experts: weights")
+    _need(pair_out.shape == (tokens * top, width) and residual.shape == (tokens, width) and weights.numel() == tokens * top,
+          "moe_experts: output shapes")
+    _i32(offsets, order, tiles, num_tiles)
+    _need(offsets.numel() == experts + 1 and order.numel() == tokens * top
+          and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts), "moe_experts: grouping")
+    fn = _fn("moe", "vk_moe_experts", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p, _p, _p])
+    _status(fn(_ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _dt(h, "h"), _ptr(offsets), _ptr(order),
+               _ptr(tiles), _ptr(num_tiles), _ptr(weights), tokens, experts, top, width, ff, float(limit), float(alpha),
+               _ptr(act), _ptr(pair_out), _ptr(residual), _stream()), "moe_experts")

@@ -2,6 +2,7 @@
 
 ``prenorm``: ``x += mixer(norm_1(x)); x += ffn(norm_2(x))``, the pre-norm residual block of the
 reference (crates/vipera-backend-cpu/src/model.rs:3-4, 975-1198).
+``parallel``: ``h = norm(x); x += mixer(h) + ffn(h)``.
 """
 from __future__ import annotations
 
@@ -71,4 +72,43 @@ class PreNormBlock(Block):
             self.ffn.forward(h, batch, x, **ffn_kwargs)
 
 
+class ParallelBlock(Block):
+    """``h = norm(x); x += mixer(h) + ffn(h)``: one norm, and both sublayers read its output.  The layer's norm is
+    ``LayerSpec.mixer_norm``; ``ffn_norm`` is not read."""
+
+    def __init__(self, spec: LayerSpec, runtime):
+        super().__init__(spec, runtime)
+        self.norm = part_class("norm", spec.mixer_norm.kind)(spec.mixer_norm, spec.prefix, runtime)
+        self.mixer = part_class("mixer", spec.mixer.kind)(spec.mixer, spec.prefix, runtime)
+        self.ffn = part_class("ffn", spec.ffn.kind)(spec.ffn, spec.prefix, runtime)
+        self.position = part_class("position", spec.position.kind)(spec.position, spec.prefix, runtime)
+
+    @classmethod
+    def _families(cls, spec: LayerSpec):
+        return (("norm", spec.mixer_norm), ("mixer", spec.mixer), ("ffn", spec.ffn), ("position", spec.position))
+
+    @classmethod
+    def declare(cls, spec: LayerSpec) -> List[TensorSpec]:
+        out: List[TensorSpec] = []
+        for family, part in cls._families(spec):
+            out += part_class(family, part.kind).declare(part, spec.prefix)
+        return out
+
+    @classmethod
+    def check_supported(cls, spec: LayerSpec, dtype) -> None:
+        for family, part in cls._families(spec):
+            part_class(family, part.kind).check_supported(part, dtype)
+
+    def load(self, tensors) -> None:
+        for part in (self.norm, self.mixer, self.ffn, self.position):
+            part.load(tensors)
+
+    def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
+        # both sublayers add into the 32-bit residual; neither reads it, so their order does not matter
+        h = self.norm.forward(x)
+        self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
+        self.ffn.forward(h, batch, x)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("parallel", ParallelBlock)

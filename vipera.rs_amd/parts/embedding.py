@@ -14,7 +14,12 @@ from ..config.base import PartSpec
 from ..ops import kernels
 from ..ops.linear import linear
 from ..weights.checkpoint import MATRIX, TensorSpec
-from .base import Part, register_embedding, register_head
+from .base import Part, part_class, register_embedding, register_head
+
+
+def _tensor_name(spec: PartSpec, prefix: str) -> str:
+    """``params["tensor"]`` names the matrix outright; otherwise it is ``<name>.weight``."""
+    return f"{prefix}{spec.params['tensor']}" if spec.params.get("tensor") else f"{prefix}{spec.params['name']}.weight"
 
 
 class Embedding(Part):
@@ -25,14 +30,29 @@ class Embedding(Part):
         self.vocab = int(spec.params["vocab"])
         self.width = int(spec.params["width"])
         self.table: Optional[torch.Tensor] = None
+        # a norm right after the table (``params["norm"]``, a PartSpec of a registered norm): the residual starts
+        # as its 32-bit output
+        norm = spec.params.get("norm")
+        self.norm = part_class("norm", norm.kind)(norm, prefix, runtime) if norm is not None else None
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
-                           (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX)]
+        specs = [TensorSpec(_tensor_name(spec, prefix), (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX)]
+        norm = spec.params.get("norm")
+        if norm is not None:
+            specs += part_class("norm", norm.kind).declare(norm, prefix)
+        return specs
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype) -> None:
+        norm = spec.params.get("norm")
+        if norm is not None:
+            part_class("norm", norm.kind).check_supported(norm, dtype)
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.table = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
+        self.table = tensors[_tensor_name(self.spec, self.prefix)]
+        if self.norm is not None:
+            self.norm.load(tensors)
 
     def embed(self, batch) -> torch.Tensor:
         """The 32-bit residual ``[tokens, width]`` a step starts from.  An embedding sees the whole batch, so one
@@ -47,6 +67,8 @@ class Embedding(Part):
         ``sampled`` on the device instead (see ``kernels.embed_gather``)."""
         out = self.runtime.empty((count, self.width), torch.float32)
         kernels.embed_gather(self.table, tokens, out, source, sampled)
+        if self.norm is not None:
+            out = self.norm.forward(out, out=self.runtime.empty((count, self.width), torch.float32))
         return out
 
 
@@ -56,18 +78,20 @@ class LMHead(Part):
         self.vocab = int(spec.params["vocab"])
         self.width = int(spec.params["width"])
         self.tied_to = spec.params.get("tied_to")
+        scale = spec.params.get("scale")
+        self.scale = float(scale) if scale is not None else 1.0     # logits = (W h) * scale
         self.weight: Optional[torch.Tensor] = None
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
         # With tied embeddings the output matrix is optional: a folder that holds one has it used, as the reference
         # uses `output.weight` whenever the file has it and the embedding table only otherwise (model.rs:424-425).
-        return [TensorSpec(f"{prefix}{spec.params['name']}.weight",
+        return [TensorSpec(_tensor_name(spec, prefix),
                            (int(spec.params["vocab"]), int(spec.params["width"])), MATRIX,
                            optional=bool(spec.params.get("tied_to")))]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        own = f"{self.prefix}{self.spec.params['name']}.weight"
+        own = _tensor_name(self.spec, self.prefix)
         if self.tied_to and own not in tensors:
             self.weight = tensors[f"{self.tied_to}.weight"]  # tied: the same buffer, no copy
         else:
@@ -76,6 +100,8 @@ class LMHead(Part):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         logits = self.runtime.empty((h.shape[0], self.vocab), torch.float32)
         linear(h, self.weight, None, logits)
+        if self.scale != 1.0:
+            kernels.scale_(logits, self.scale)
         return logits
 
 

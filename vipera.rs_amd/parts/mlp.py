@@ -80,4 +80,12 @@ class GatedMLP(FeedForward):
             linear(act, self.w_down, None, residual, accumulate=True)
 
 
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: adds nothing."""
+
+    def forward(self, h, batch, residual, **_unused) -> None:
+        return None
+
+
 register_ffn("gated_mlp", GatedMLP)
+register_ffn("none", NoFeedForward)

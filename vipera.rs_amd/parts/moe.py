@@ -1,0 +1,87 @@
+"""Mixture of experts: each token runs ``top`` of ``experts`` small gated feed-forwards.
+
+Router logits ``z = W_router h`` in 32-bit; the ``top`` largest are chosen (the lowest id among equals) and weighted
+by the softmax over the chosen logits only.  An expert computes ``g = min(W_gate h, limit)``,
+``u = clamp(W_up h, -limit, limit)``, ``y = g * sigmoid(alpha * g) * (u + 1)`` and returns ``W_down y``; the layer
+adds the weighted sum of the chosen experts' outputs to the residual.  ``limit`` and ``alpha`` are parameters.
+
+The step's (token, choice) pairs are grouped by expert on the device, so nothing about the routing reaches the
+host and a step of single tokens can be captured; see ``csrc/kernels/moe.hip``.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from ..config.base import PartSpec
+from ..errors import InvalidArgumentError, UnsupportedError
+from ..ops import kernels
+from ..ops.linear import linear
+from ..weights.checkpoint import MATRIX, TensorSpec
+from .base import FeedForward, register_ffn
+
+
+class MixtureOfExperts(FeedForward):
+    """``params``: ``hidden``, ``intermediate`` (an expert's width), ``experts``, ``top``, ``limit``, ``alpha``
+    (1.702 unless given), ``name``; tensors ``<name>.router`` and ``<name>.e<i>.gate | up | down``."""
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.inter = int(p["hidden"]), int(p["intermediate"])
+        self.experts, self.top = int(p["experts"]), int(p["top"])
+        self.limit = float(p["limit"])
+        self.alpha = float(p.get("alpha", 1.702))
+        if not 1 <= self.top <= self.experts:
+            raise InvalidArgumentError(f"a token cannot use {self.top} of {self.experts} experts")
+        self.w_router = self.w_gate = self.w_up = self.w_down = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, inter = int(p["hidden"]), int(p["intermediate"])
+        specs = []
+        for e in range(int(p["experts"])):
+            specs += [TensorSpec(f"{base}e{e}.gate", (inter, hidden), MATRIX),
+                      TensorSpec(f"{base}e{e}.up", (inter, hidden), MATRIX),
+                      TensorSpec(f"{base}e{e}.down", (hidden, inter), MATRIX)]
+        specs.append(TensorSpec(base + "router", (int(p["experts"]), hidden), MATRIX))
+        return specs
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        experts, top = int(spec.params["experts"]), int(spec.params["top"])
+        if top > 64 or experts > 4096:
+            raise UnsupportedError(f"mixture of experts: top {top} of {experts} experts is above the routing kernel's "
+                                   "limits of 64 of 4,096")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        dtype = self.runtime.dtype
+        stack = lambda kind: torch.stack([tensors[f"{base}e{e}.{kind}"].to(dtype) for e in range(self.experts)]).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        self.w_router = tensors[base + "router"]
+
+    def forward(self, h, batch, residual, **_unused) -> None:
+        tokens = residual.shape[0]
+        device = residual.device
+        pairs = tokens * self.top
+        logits = torch.empty((tokens, self.experts), dtype=torch.float32, device=device)
+        linear(h, self.w_router, None, logits)
+        ints = torch.empty(2 * pairs + self.experts + 2 + 2 * kernels.moe_max_tiles(pairs, self.experts),
+                           dtype=torch.int32, device=device)
+        ids, order = ints[:pairs], ints[pairs:2 * pairs]
+        offsets = ints[2 * pairs:2 * pairs + self.experts + 1]
+        num_tiles = ints[2 * pairs + self.experts + 1:2 * pairs + self.experts + 2]
+        tiles = ints[2 * pairs + self.experts + 2:]
+        weights = torch.empty(pairs, dtype=torch.float32, device=device)
+        kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles)
+        act = self.runtime.empty((pairs, self.inter))
+        pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
+        kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,
+                            self.top, self.limit, self.alpha, act, pair_out, residual)
+
+
+register_ffn("moe", MixtureOfExperts)

@@ -1,4 +1,4 @@
-"""RMSNorm: ``out = (x * rsqrt(mean(x^2) + eps)) * weight`` with the sum in 32-bit.
+"""Norms.  RMSNorm: ``out = (x * rsqrt(mean(x^2) + eps)) * weight`` with the sum in 32-bit; Dynamic Tanh below.
 
 Reference: crates/vipera-backend-cpu/src/model.rs:4282-4288 (eps inside the square root, added to
 the mean; multiply order ``(x * inv) * w``).
@@ -45,4 +45,36 @@ class RMSNorm(Norm):
         return out
 
 
+class DynamicTanh(Norm):
+    """Dynamic Tanh: ``out = tanh(alpha * x) * weight + bias`` per element, with one learned number ``alpha``; no
+    mean and no variance is computed (Zhu, Chen, He, LeCun, Liu: "Transformers without Normalization").  Tensors:
+    ``<name>`` (the weight), ``<name>.alpha`` and ``<name>.b``; ``params["name"]`` is the weight's name after the
+    part's prefix."""
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        self.width = int(spec.params["width"])
+        self.weight = self.bias = self.alpha = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        name, width = f"{prefix}{spec.params['name']}", int(spec.params["width"])
+        return [TensorSpec(name, (width,), VECTOR, "one_plus_normal"),
+                TensorSpec(name + ".b", (width,), VECTOR, "normal"),
+                TensorSpec(name + ".alpha", (), VECTOR, "one_plus_normal")]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        name = f"{self.prefix}{self.spec.params['name']}"
+        self.weight, self.bias = tensors[name], tensors[name + ".b"]
+        self.alpha = tensors[name + ".alpha"].reshape(1)
+
+    def forward(self, x, out=None, rows=None):
+        count = x.shape[0] if rows is None else rows.numel()
+        if out is None:
+            out = self.runtime.empty((count, self.width))
+        kernels.dyt(x, self.alpha, self.weight, self.bias, out, rows)
+        return out
+
+
 register_norm("rmsnorm", RMSNorm)
+register_norm("dyt", DynamicTanh)

@@ -1,0 +1,199 @@
+"""Recurrent mixers: layers that keep a matrix of state per head instead of a cache of keys and values.
+
+``gated_delta``: the gated delta rule.  ``q = Wq h``, ``k = Wk h`` (``kv_heads x dim``), ``v = Wv h``
+(``heads x vdim``); each passes a short causal convolution over time per channel and silu; q and k become unit
+vectors per head (q also times ``dim^-1/2``); ``beta = sigmoid(Wb h)``, ``g = exp(-exp(A_log) softplus(Wa h +
+dt_bias))`` per head; then per head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``; the read-out is
+``o / rms(o) * norm * silu(Wg h)`` and goes through ``Wo``.
+
+``wkv``: RWKV-style time mixing.  Each of r, k, v, g, w reads its own mix ``h + (h_prev - h) * mu``; the decay is
+``w = exp(-exp(W2 tanh(W1 mix_w) + w0))`` per key channel; per head ``o = (S + diag(u) k v^T)^T r`` and then
+``S <- diag(w) S + k v^T``; the read-out is ``o / rms(o) * norm * silu(Wg mix_g)`` and goes through ``Wo``.
+
+Both keep their state in 32-bit in the request's slot: the matrices, and what the next token needs of this one (the
+convolution's last inputs; the last ``h``).  An entry that starts at position 0 starts from zeros.  Everything the
+kernels look at lies on the device, so a step of single tokens can be captured.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from ..config.base import PartSpec
+from ..errors import InvalidArgumentError, UnsupportedError
+from ..ops import kernels
+from ..ops.linear import linear
+from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
+from .attention import _cat
+from .base import Mixer, StateSpec, register_mixer
+
+UNIT_EPS = 1e-6   # q and k of the delta rule: x / sqrt(sum(x^2) + UNIT_EPS)
+
+
+class GatedDelta(Mixer):
+    """``params``: ``hidden``, ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``conv`` (taps), ``eps`` (of the read-out's
+    norm), ``name``."""
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.heads, self.kv_heads = int(p["hidden"]), int(p["heads"]), int(p["kv_heads"])
+        self.dim, self.vdim, self.taps = int(p["dim"]), int(p["vdim"]), int(p["conv"])
+        self.eps = float(p["eps"])
+        if self.heads % self.kv_heads:
+            raise InvalidArgumentError(f"heads {self.heads} is not a multiple of kv_heads {self.kv_heads}")
+        self.qk, self.vw = self.kv_heads * self.dim, self.heads * self.vdim
+        self.channels = 2 * self.qk + self.vw
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+
+    @classmethod
+    def _sizes(cls, p):
+        qk, vw = int(p["kv_heads"]) * int(p["dim"]), int(p["heads"]) * int(p["vdim"])
+        return qk, vw, 2 * qk + vw
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, heads, taps = int(p["hidden"]), int(p["heads"]), int(p["conv"])
+        qk, vw, _ = cls._sizes(p)
+        specs = []
+        for name, rows in (("q", qk), ("k", qk), ("v", vw)):
+            specs.append(TensorSpec(base + name, (rows, hidden), MATRIX))
+            specs.append(TensorSpec(f"{base}{name}.conv", (rows, taps), VECTOR, std=0.5))
+        specs += [TensorSpec(base + "b", (heads, hidden), MATRIX), TensorSpec(base + "A_log", (heads,), VECTOR),
+                  TensorSpec(base + "norm", (int(p["vdim"]),), VECTOR, "one_plus_normal"),
+                  TensorSpec(base + "a", (heads, hidden), MATRIX), TensorSpec(base + "dt_bias", (heads,), VECTOR),
+                  TensorSpec(base + "g", (vw, hidden), MATRIX), TensorSpec(base + "o", (hidden, vw), MATRIX)]
+        return specs
+
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        p = spec.params
+        _, _, channels = cls._sizes(p)
+        floats = int(p["heads"]) * int(p["dim"]) * int(p["vdim"]) + (int(p["conv"]) - 1) * channels
+        return None, StateSpec((floats,), torch.float32)
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        p = spec.params
+        if int(p["dim"]) > kernels.RECURRENT_MAX_KEY_DIM:
+            raise UnsupportedError(f"gated_delta: a key width of {p['dim']} is above the kernel's limit of "
+                                   f"{kernels.RECURRENT_MAX_KEY_DIM}")
+        if int(p["conv"]) < 1:
+            raise UnsupportedError(f"gated_delta: the convolution needs at least one tap, got {p['conv']}")
+        if cls._sizes(p)[2] > 16_384:
+            raise UnsupportedError("gated_delta: more than 16,384 convolved channels do not fit the kernel's LDS row")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        # one product for everything that reads h: [q | k | v | g | b | a] rows
+        self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", "g", "b", "a")])
+        self.conv = torch.cat([tensors[f"{base}{n}.conv"] for n in ("q", "k", "v")]).contiguous()
+        self.a_log, self.dt_bias, self.norm = tensors[base + "A_log"], tensors[base + "dt_bias"], tensors[base + "norm"]
+        self.w_o = tensors[base + "o"]
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+        tokens, entries = residual.shape[0], batch.num_entries
+        device = residual.device
+        f32 = dict(dtype=torch.float32, device=device)
+        # what enters the recurrence stays 32-bit from the product's sums on
+        proj = torch.empty((tokens, self.w_in.shape[0]), **f32)
+        linear(h, self.w_in, None, proj)
+        qkv = torch.empty((tokens, self.channels), **f32)
+        beta, decay = torch.empty((tokens, self.heads), **f32), torch.empty((tokens, self.heads), **f32)
+        g_col = self.channels
+        b_col = g_col + self.vw
+        matrices = self.heads * self.dim * self.vdim
+        kernels.delta_prepare(proj, self.conv, state, matrices, batch.entry_of_token, batch.entry_start,
+                              batch.entry_first_pos, batch.slots, self.a_log, self.dt_bias, self.kv_heads, self.dim,
+                              self.heads, self.vdim, b_col, b_col + self.heads, UNIT_EPS, qkv, beta, decay, entries)
+        o = torch.empty((tokens, self.vw), **f32)
+        kernels.delta_rule(qkv, beta, decay, state, batch.entry_start, batch.entry_first_pos, batch.slots,
+                           self.kv_heads, self.dim, self.heads, self.vdim, o, entries)
+        gated = self.runtime.empty((tokens, self.vw))
+        kernels.head_norm_gate(o, self.norm, proj[:, g_col:g_col + self.vw], True, self.eps, self.heads, self.vdim, gated)
+        linear(gated, self.w_o, None, residual, accumulate=True)
+
+
+class Wkv(Mixer):
+    """``params``: ``hidden``, ``heads``, ``dim``, ``eps``, ``name``, and ``decay_rank`` (rows of W1; 0 or absent: as many
+    as the folder's tensor has)."""
+
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.heads, self.dim = int(p["hidden"]), int(p["heads"]), int(p["dim"])
+        self.rank, self.eps = int(p.get("decay_rank") or 0), float(p["eps"])
+        self.width = self.heads * self.dim
+        self.mu = self.w = self.w1 = self.w2 = self.w0 = self.bonus = self.norm = self.w_o = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, heads, dim, rank = int(p["hidden"]), int(p["heads"]), int(p["dim"]), int(p.get("decay_rank") or 0) or -1
+        width = heads * dim
+        specs = [TensorSpec(f"{base}mu.{s}", (hidden,), VECTOR, std=0.3) for s in cls.MIXES]
+        specs += [TensorSpec(base + "k", (width, hidden), MATRIX), TensorSpec(base + "v", (width, hidden), MATRIX),
+                  TensorSpec(base + "g", (width, hidden), MATRIX), TensorSpec(base + "w1", (rank, hidden), MATRIX),
+                  TensorSpec(base + "w2", (width, rank), MATRIX), TensorSpec(base + "w0", (width,), VECTOR),
+                  TensorSpec(base + "u", (heads, dim), VECTOR), TensorSpec(base + "norm", (width,), VECTOR, "one_plus_normal"),
+                  TensorSpec(base + "o", (hidden, width), MATRIX), TensorSpec(base + "r", (width, hidden), MATRIX)]
+        return specs
+
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        p = spec.params
+        return None, StateSpec((int(p["heads"]) * int(p["dim"]) ** 2 + int(p["hidden"]),), torch.float32)
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        if int(spec.params["dim"]) > kernels.RECURRENT_MAX_KEY_DIM:
+            raise UnsupportedError(f"wkv: a head width of {spec.params['dim']} is above the kernel's limit of "
+                                   f"{kernels.RECURRENT_MAX_KEY_DIM}")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        self.mu = torch.stack([tensors[f"{base}mu.{s}"] for s in self.MIXES]).contiguous()
+        self.w = {s: tensors[base + s] for s in ("r", "k", "v", "g")}
+        self.w1, self.w2 = tensors[base + "w1"], tensors[base + "w2"]
+        self.rank = int(self.w1.shape[0])
+        if self.w2.shape[1] != self.rank:
+            raise InvalidArgumentError(f"{base}w2 has {self.w2.shape[1]} columns for the {self.rank} rows of {base}w1")
+        self.w0, self.bonus = tensors[base + "w0"], tensors[base + "u"].reshape(-1).contiguous()
+        self.norm, self.w_o = tensors[base + "norm"], tensors[base + "o"]
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+        tokens, entries = residual.shape[0], batch.num_entries
+        device = residual.device
+        f32 = dict(dtype=torch.float32, device=device)
+        matrices = self.heads * self.dim * self.dim
+        mixes = self.runtime.empty((len(self.MIXES), tokens, self.hidden))
+        kernels.token_shift(h, self.mu, state, matrices, batch.entry_of_token, batch.entry_start,
+                            batch.entry_first_pos, batch.slots, mixes, entries)
+        # r, k, v and the decay enter the recurrence: 32-bit from their products' sums on
+        rkv = torch.empty((3, tokens, self.width), **f32)
+        for index, name in enumerate(("r", "k", "v")):
+            linear(mixes[index], self.w[name], None, rkv[index])
+        gate = self.runtime.empty((tokens, self.width))
+        linear(mixes[3], self.w["g"], None, gate)
+        low = torch.empty((tokens, self.rank), **f32)
+        linear(mixes[4], self.w1, None, low)
+        squashed = torch.empty((tokens, self.rank), **f32)
+        kernels.tanh(low, squashed)
+        wraw = torch.empty((tokens, self.width), **f32)
+        linear(squashed, self.w2, None, wraw)
+        o = torch.empty((tokens, self.width), **f32)
+        kernels.wkv_rule(rkv[0], rkv[1], rkv[2], wraw, self.w0, self.bonus, state, batch.entry_start,
+                         batch.entry_first_pos, batch.slots, self.dim, self.heads, o, entries)
+        gated = self.runtime.empty((tokens, self.width))
+        kernels.head_norm_gate(o, self.norm, gate, True, self.eps, self.heads, self.dim, gated)
+        linear(gated, self.w_o, None, residual, accumulate=True)
+
+
+register_mixer("gated_delta", GatedDelta)
+register_mixer("wkv", Wkv)

@@ -28,7 +28,7 @@ class TensorSpec:
     """A tensor that a part needs: its name, shape, how it is kept, and how random weights fill it."""
 
     name: str
-    shape: Tuple[int, ...]
+    shape: Tuple[int, ...]    # a dimension of -1 is whatever the folder stores (a size that no configuration key gives)
     role: str = MATRIX
     init: str = "normal"      # "normal" N(0, std) | "one_plus_normal" 1 + N(0, std) | "zeros" | "ones"
     std: float = 0.02
@@ -112,8 +112,9 @@ class Checkpoint:
         for name, spec in wanted.items():
             if name in self.tensors:
                 found = self.tensors[name][1].shape
-                if tuple(found) != tuple(spec.shape):
-                    wrong.append((name, tuple(found), tuple(spec.shape)))
+                want = tuple(spec.shape)
+                if len(found) != len(want) or any(w != -1 and int(f) != int(w) for f, w in zip(found, want)):
+                    wrong.append((name, tuple(found), want))
         if missing or unexpected or wrong:
             raise WeightsError(self.folder, missing, unexpected, wrong)
 
@@ -151,8 +152,8 @@ def kept_bytes(checkpoint: Checkpoint, specs: Sequence[TensorSpec], run_dtype: t
         if not present and spec.optional:
             continue
         count = 1
-        for dim in spec.shape:
-            count *= int(dim)
+        for dim in (checkpoint.info(spec.name).shape if present else spec.shape):
+            count *= max(int(dim), 0)
         stored = checkpoint.info(spec.name).torch_dtype if present else run_dtype
         total += count * torch.empty(0, dtype=kept_dtype(spec, stored, run_dtype, keep_float32)).element_size()
     return total

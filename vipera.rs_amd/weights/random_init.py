@@ -52,6 +52,8 @@ def standard_normal(key: int, count: int) -> np.ndarray:
 
 
 def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tensor:
+    if any(int(dim) < 0 for dim in spec.shape):
+        raise ValueError(f"tensor \"{spec.name}\": a size is left to the model's files; random weights need it in the configuration")
     count = 1
     for dim in spec.shape:
         count *= dim
