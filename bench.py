@@ -106,6 +106,11 @@ def main() -> int:
                         help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
                              "pair of GPU events around every kernel launch, and add the microseconds of each class of "
                              "kernel to the line (split_decode_us, split_prefill_us)")
+    parser.add_argument("--design", default="", choices=["", "gilidra"],
+                        help="instead of the headline measurement: prefill and decode of this design at layer sizes that "
+                             "resemble a real model's (--size), beside the dense Qwen2 decoder of the same width, depth and "
+                             "active feed-forward width, each with the time of every class of kernel")
+    parser.add_argument("--size", default="m", choices=["s", "m"], help="with --design: the layer sizes (see DESIGN_SIZES)")
     parser.add_argument("--in-turn", action="store_true",
                         help="wait for a step's tokens on the host before the next step is launched")
     args = parser.parse_args()
@@ -114,6 +119,8 @@ def main() -> int:
         return 2
 
     still_running()
+    if args.design:
+        return design_comparison(args)
 
     import torch
 
@@ -350,6 +357,134 @@ def kernel_split(args, config, runner, tokens, ctx, T):
     log("split of one decode step (us): " + ", ".join(f"{k} {v}" for k, v in decode.items()))
     log("split of one prefill (us): " + ", ".join(f"{k} {v}" for k, v in prefill.items()))
     return {"split_decode_us": decode, "split_prefill_us": prefill}
+
+
+# Layer sizes for --design: (width, layers, vocab, attention heads, key width, latent ranks (q, kv), rotated dims,
+# delta heads / key heads, wkv heads, experts, top, an expert's width).  The cached row of a latent layer is
+# kv_rank + rot_dim = 256 wide, the attention kernels' limit.
+DESIGN_SIZES = {
+    "s": dict(width=1024, layers=10, vocab=32768, heads=8, dim=128, q_rank=384, kv_rank=192, rot=64, delta_heads=8,
+              delta_kv=4, wkv_heads=16, experts=16, top=4, ff=512, window=1024),
+    "m": dict(width=2048, layers=10, vocab=65536, heads=16, dim=128, q_rank=768, kv_rank=192, rot=64, delta_heads=16,
+              delta_kv=8, wkv_heads=32, experts=32, top=4, ff=1024, window=2048),
+}
+
+
+def gilidra_shape(z):
+    """A Gilidra configuration of sizes ``z``: latent attention, delta rule, time mixing, a latent layer that reads the
+    first one's cache, delta rule, and so on; a mixture of experts beside every mixer."""
+    moe = {"kind": "moe", "expert": {"ff": z["ff"], "limit": 7.0}, "router": {"experts": z["experts"], "top": z["top"]}}
+    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot"], "vdim": z["dim"], "q_rank": z["q_rank"],
+              "kv_rank": z["kv_rank"], "rot": {"base": 1e6, "dims": z["rot"]}, "scale": (z["dim"] + z["rot"]) ** -0.5,
+              "mask": {"size": z["window"]}}
+    layers = []
+    for index in range(z["layers"]):
+        kind = index % 5
+        if kind in (0, 3):
+            mixer = dict(latent, kv_from=index - 3) if kind == 3 else dict(latent)
+            layers.append({"type": "latent_attention", "mixer": mixer, "mlp": moe})
+        elif kind in (1, 4):
+            layers.append({"type": "delta", "mlp": moe, "mixer": {"heads": z["delta_heads"], "kv_heads": z["delta_kv"],
+                                                                 "dim": 128, "vdim": 128, "conv": 4}})
+        else:
+            layers.append({"type": "wkv", "mlp": moe, "mixer": {"heads": z["wkv_heads"], "dim": 64, "decay_rank": 64}})
+    return {"architecture": "Gilidra", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
+            "logit_scale": 1.0, "layers": layers}
+
+
+def dense_shape(z):
+    """The dense Qwen2 decoder of the same width, depth, heads and active feed-forward width."""
+    return dict(QWEN25_7B, num_hidden_layers=z["layers"], hidden_size=z["width"], num_attention_heads=z["heads"],
+                num_key_value_heads=max(1, z["heads"] // 4), head_dim=z["dim"], intermediate_size=z["top"] * z["ff"],
+                vocab_size=z["vocab"], max_window_layers=z["layers"])
+
+
+def design_comparison(args) -> int:
+    """Prefill (one prompt of --prefill-tokens) and decode (batches --batch and --points at context --ctx) of the
+    design and of the dense decoder of equal size, eagerly for the time of every class of kernel and as the engine
+    runs them (captured decode steps) for the throughput."""
+    import torch
+
+    import vipera_rs_amd  # noqa: F401
+    from vipera_rs_amd.config import config_from_dict
+    from vipera_rs_amd.engine.batch import StepEntry
+    from vipera_rs_amd.engine.runner import ModelRunner
+    from vipera_rs_amd.models import build_model
+    from vipera_rs_amd.ops import profile
+    from vipera_rs_amd.runtime import Runtime
+    from vipera_rs_amd.weights import random_device_tensors
+
+    z = DESIGN_SIZES[args.size]
+    T, ctx = args.prefill_tokens, args.ctx
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
+    largest = max(batches)
+    gen = torch.Generator().manual_seed(0)
+    out = {}
+    for name, shape in (("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))):
+        config = config_from_dict(shape)
+        runtime = Runtime("cuda:0", args.dtype)
+        model = build_model(config, runtime)
+        model.load(random_device_tensors(model.tensor_specs(), 0, runtime.dtype, runtime.device))
+        pages = largest * ((ctx + 64 + args.block_size - 1) // args.block_size) + T // args.block_size + 8
+        runner = ModelRunner(model, runtime, args.block_size, pages, largest + 1, use_graphs=True, max_context=ctx + 64)
+        prompt = torch.randint(0, config.vocab_size, (T,), generator=gen).tolist()
+
+        def label(binding, call_args, call_kwargs):
+            shape_of = profile.weight_shape(binding, call_args)
+            return f"{binding} {shape_of[0]}x{shape_of[1]}" if shape_of else binding
+
+        def prefill(request):
+            runner.cache.reserve(request, 0, T)
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            runner.step([StepEntry(request, 0, prompt, [T - 1])])
+            torch.cuda.synchronize()
+            seconds = time.perf_counter() - started
+            runner.cache.release(request)
+            return seconds
+
+        prefill(0)
+        prefill_s = min(prefill(1 + k) for k in range(3))
+        with profile.KernelTimer(label) as timer:
+            timer.hold_back()
+            prefill(5)
+        result = {"prefill_ms": round(prefill_s * 1e3, 3), "prefill_tok_s": round(T / prefill_s, 1),
+                  "prefill_us_by_kernel": {k: round(v, 1) for k, v in sorted(timer.microseconds().items())}}
+        log(f"{name}: prefill of {T} tokens {result['prefill_ms']} ms, {result['prefill_tok_s']} tokens/s")
+        for batch in batches:
+            # decode steps at context ctx: the cache's pages hold nothing a prompt wrote, and a recurrent layer's
+            # state rows are zeros; no kernel's time depends on either
+            for request in range(batch):
+                runner.cache.reserve(100 + request, 0, ctx + 40)
+            def step(k):
+                return runner.step([StepEntry(100 + r, ctx + k, [1 + r], [0]) for r in range(batch)])
+            for k in range(4):
+                step(k)
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            for k in range(4, 4 + args.steps // 2):
+                step(k)
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - started) / (args.steps // 2) * 1e3
+            result[f"decode_b{batch}_ms"] = round(ms, 4)
+            result[f"decode_b{batch}_tok_s"] = round(batch / ms * 1e3, 1)
+            if batch == args.batch:
+                graphs, runner.graphs = runner.graphs, None
+                with profile.KernelTimer(label) as timer:
+                    timer.hold_back()
+                    step(36)
+                runner.graphs = graphs
+                result[f"decode_b{batch}_us_by_kernel"] = {k: round(v, 1) for k, v in sorted(timer.microseconds().items())}
+            for request in range(batch):
+                runner.cache.release(100 + request)
+            log(f"{name}: decode batch {batch} at context {ctx}: {ms:.3f} ms a step, {batch / ms * 1e3:.0f} tokens/s")
+        out[name] = result
+        del runner, model
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": f"prefill and decode of {args.design} beside the dense decoder of equal size",
+                      "size": z, "dtype": args.dtype, "prefill_tokens": T, "ctx": ctx, "data": "synthetic: seeded random "
+                      "weights and uniform-random token ids", **out}), flush=True)
+    return 0
 
 
 def serving(args, config, runtime, model, shape_name, layers_full, dtype_key) -> int:

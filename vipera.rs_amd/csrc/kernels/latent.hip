@@ -8,6 +8,7 @@
 // through Wuv_h.  The cache holds the row twice, as keys [page, 1, slot, rank + rot] and transposed as values
 // [page, 1, rank + rot, slot], which is the layout the paged attention kernels read.
 #include "common.h"
+#include "group_tile.h"
 
 // ---------------------------------------------------------------------------------------------
 // One workgroup per token: c = rms_norm(x[:rank]) * weight, kr = rotate(x[rank:]) (pairs (i, i + rot_dims / 2) of
@@ -134,6 +135,35 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TA* __restrict__
   }
 }
 
+// The same product on the matrix cores (bfloat16 in and out; K a multiple of 8, 16-byte rows): tiles of 128 tokens
+// x 128 outputs of one head, see group_tile.h.  Grid (ceil(T / 128), ceil(N / 128), heads).
+__global__ __launch_bounds__(256) void head_linear_mma_kernel(const __bf16* __restrict__ a, long long lda, long long sa,
+                                                              const __bf16* __restrict__ w, __bf16* __restrict__ out,
+                                                              long long ldo, long long so, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int h = blockIdx.z, m0 = blockIdx.x * GT_TILE, n0 = blockIdx.y * GT_TILE;
+  const __bf16* ah = a + (long long)h * sa;
+  const __bf16* wh = w + (long long)h * N * K;
+  gt_f32x4 acc[4][4];
+  group_tile_mma([&](int r) -> const __bf16* { return m0 + r < M ? ah + (long long)(m0 + r) * lda : nullptr; },
+                 [&](int r) -> const __bf16* { return n0 + r < N ? wh + (long long)(n0 + r) * K : nullptr; }, K, lds, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 15, lg = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const int m = m0 + wm * 64 + tm * 16 + lr;
+    if (m >= M) continue;
+    __bf16* dst = out + (long long)m * ldo + (long long)h * so;
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + wn * 64 + tn * 16 + lg * 4 + i;
+        if (n < N) dst[n] = (__bf16)acc[tn][tm][i];
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 extern "C" int vk_latent_kv_write(const float* x, long long ldx, const float* weight, float eps, int rank, int rot,
                                   int rot_dims, const int* positions, const float* inv_freq, const int* entry_of,
@@ -189,7 +219,19 @@ extern "C" int vk_head_linear(const void* a, int a_dtype, long long lda, long lo
   if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32)
     head_linear_kernel<float, float, float><<<grid, 256, 0, s>>>((const float*)a, lda, sa, (const float*)w, (float*)out,
                                                                  ldo, so, M, N, K);
-  else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16)
+  else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16 && K % 8 == 0 && lda % 8 == 0 && sa % 8 == 0 &&
+           (((uintptr_t)a | (uintptr_t)w) & 15) == 0) {
+    static bool sized = false;
+    if (!sized) {
+      hipError_t e = hipFuncSetAttribute((const void*)head_linear_mma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         GT_LDS_BYTES);
+      if (e != hipSuccess) return (int)e;
+      sized = true;
+    }
+    dim3 wide((M + GT_TILE - 1) / GT_TILE, (N + GT_TILE - 1) / GT_TILE, heads);
+    head_linear_mma_kernel<<<wide, 256, GT_LDS_BYTES, s>>>((const __bf16*)a, lda, sa, (const __bf16*)w, (__bf16*)out, ldo,
+                                                           so, M, N, K);
+  } else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16)
     head_linear_kernel<bf16_t, bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a, lda, sa, (const bf16_t*)w,
                                                                     (bf16_t*)out, ldo, so, M, N, K);
   else if (a_dtype == DT_BF16 && w_dtype == DT_F32 && out_dtype == DT_BF16)

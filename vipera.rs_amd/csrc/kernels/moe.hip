@@ -8,8 +8,9 @@
 // but no value does: a pair's row is computed alone, an FMA chain in k order per output element, and the
 // weighted sum over a token's choices runs in the order of the choices.
 #include "common.h"
+#include "group_tile.h"
 
-constexpr int MOE_TILE = 64;
+constexpr int MOE_TILE = 64;      // places per tile of the 32-bit products; the matrix-core products take 128
 
 // ---------------------------------------------------------------------------------------------
 // One wave per token: the `top` largest of E logits (the lowest id wins a tie), and the softmax over those.
@@ -56,8 +57,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 // One workgroup: counts per expert, offsets, the pairs' places, and the list of tiles.
 //   offsets [E + 1], order [P], tiles [max_tiles][2] = (expert, first place), num_tiles [1]
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int pairs, int experts,
-                                                         int* __restrict__ offsets, int* __restrict__ order,
-                                                         int* __restrict__ tiles, int* __restrict__ num_tiles) {
+                                                         int tile_rows, int* __restrict__ offsets,
+                                                         int* __restrict__ order, int* __restrict__ tiles,
+                                                         int* __restrict__ num_tiles) {
   extern __shared__ int shared[];      // counts [E], cursor [E]
   int* counts = shared;
   int* cursor = shared + experts;
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
     for (int e = 0; e < experts; ++e) {
       offsets[e] = at;
       cursor[e] = at;
-      for (int first = 0; first < counts[e]; first += MOE_TILE) {
+      for (int first = 0; first < counts[e]; first += tile_rows) {
         tiles[2 * tile] = e;
         tiles[2 * tile + 1] = at + first;
         ++tile;
@@ -203,6 +205,89 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same two products on the matrix cores (bfloat16): tiles of 128 places, see group_tile.h.  A workgroup of the
+// gate/up product owns 64 columns of an expert's width: each wave holds gate and up of the same 32 columns.
+__global__ __launch_bounds__(256) void moe_gate_up_mma_kernel(const __bf16* __restrict__ h, long long ldh,
+                                                              const __bf16* __restrict__ wg,
+                                                              const __bf16* __restrict__ wu,
+                                                              const int* __restrict__ offsets,
+                                                              const int* __restrict__ order,
+                                                              const int* __restrict__ tiles,
+                                                              const int* __restrict__ num_tiles, int top, int width,
+                                                              int ff, float limit, float alpha,
+                                                              __bf16* __restrict__ act) {
+  if ((int)blockIdx.x >= num_tiles[0]) return;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  __shared__ int rows[GT_TILE];
+  const int e = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
+  const int count = min(GT_TILE, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * 64;
+  for (int i = threadIdx.x; i < GT_TILE; i += 256) rows[i] = i < count ? order[first + i] / top : -1;
+  __syncthreads();
+  const __bf16* g_w = wg + (long long)e * ff * width;
+  const __bf16* u_w = wu + (long long)e * ff * width;
+  gt_f32x4 acc[4][4];
+  group_tile_mma(
+      [&](int r) -> const __bf16* { return rows[r] >= 0 ? h + (long long)rows[r] * ldh : nullptr; },
+      [&](int r) -> const __bf16* {
+        const int col = n0 + (r >> 6) * 32 + ((r >> 4) & 1) * 16 + (r & 15);
+        if (col >= ff) return nullptr;
+        return (((r >> 5) & 1) ? u_w : g_w) + (long long)col * width;
+      },
+      width, lds, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 15, lg = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const int r = wm * 64 + tm * 16 + lr;
+    if (r >= count) continue;
+#pragma unroll
+    for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int col = n0 + wn * 32 + tn * 16 + lg * 4 + i;
+        if (col >= ff) continue;
+        const float g = fminf(acc[tn][tm][i], limit);
+        const float u = fminf(fmaxf(acc[tn + 2][tm][i], -limit), limit);
+        act[(long long)(first + r) * ff + col] = (__bf16)(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+      }
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_down_mma_kernel(const __bf16* __restrict__ act, const __bf16* __restrict__ wd,
+                                                           const int* __restrict__ offsets,
+                                                           const int* __restrict__ order,
+                                                           const int* __restrict__ tiles,
+                                                           const int* __restrict__ num_tiles, int width, int ff,
+                                                           float* __restrict__ pair_out) {
+  if ((int)blockIdx.x >= num_tiles[0]) return;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int e = tiles[2 * blockIdx.x], first = tiles[2 * blockIdx.x + 1];
+  const int count = min(GT_TILE, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * GT_TILE;
+  const __bf16* w = wd + (long long)e * width * ff;
+  gt_f32x4 acc[4][4];
+  group_tile_mma([&](int r) -> const __bf16* { return r < count ? act + (long long)(first + r) * ff : nullptr; },
+                 [&](int r) -> const __bf16* { return n0 + r < width ? w + (long long)(n0 + r) * ff : nullptr; }, ff,
+                 lds, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 15, lg = lane >> 4;
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const int r = wm * 64 + tm * 16 + lr;
+    if (r >= count) continue;
+    float* dst = pair_out + (long long)order[first + r] * width;
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int col = n0 + wn * 64 + tn * 16 + lg * 4 + i;
+        if (col < width) dst[col] = acc[tn][tm][i];
+      }
+  }
+}
+
 // residual[t, :] += sum_j weights[t, j] * pair_out[t * top + j, :], j ascending.
 __global__ void moe_combine_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, int top,
                                    int width, long long total, float* __restrict__ residual) {
@@ -216,10 +301,22 @@ __global__ void moe_combine_kernel(const float* __restrict__ pair_out, const flo
 }
 
 // ---------------------------------------------------------------------------------------------
-extern "C" int vk_moe_max_tiles(int pairs, int experts) { return (pairs + MOE_TILE - 1) / MOE_TILE + experts; }
+extern "C" int vk_moe_max_tiles(int pairs, int experts, int tile_rows) {
+  return (pairs + tile_rows - 1) / tile_rows + experts;
+}
 
-extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int* ids, float* weights,
-                            int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+// Whether the products of these operands run on the matrix cores (tiles of 128 places) or as 32-bit FMAs (64).
+static inline bool moe_on_matrix_cores(int dtype, int width, int ff, long long ldh) {
+  return dtype == DT_BF16 && width % 8 == 0 && ff % 8 == 0 && ldh % 8 == 0;
+}
+
+extern "C" int vk_moe_tile_rows(int dtype, int width, int ff, long long ldh) {
+  return moe_on_matrix_cores(dtype, width, ff, ldh) ? GT_TILE : MOE_TILE;
+}
+
+extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int tile_rows, int* ids,
+                            float* weights, int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+  if (tile_rows != MOE_TILE && tile_rows != GT_TILE) return VK_BAD_ARGUMENT;
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
@@ -228,8 +325,8 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
   VK_LAUNCH_CHECK();
   const long long pairs = (long long)num_tokens * top;
   if (pairs > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
-  moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(ids, (int)pairs, experts, offsets, order, tiles,
-                                                                       num_tiles);
+  moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(ids, (int)pairs, experts, tile_rows, offsets,
+                                                                       order, tiles, num_tiles);
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -241,8 +338,32 @@ extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, cons
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || width < 1 || ff < 1) return VK_BAD_ARGUMENT;
   const int pairs = num_tokens * top;
-  const int max_tiles = vk_moe_max_tiles(pairs, experts);
   hipStream_t s = (hipStream_t)stream;
+  if (moe_on_matrix_cores(dtype, width, ff, ldh)) {
+    if (((uintptr_t)h | (uintptr_t)wg | (uintptr_t)wu | (uintptr_t)wd | (uintptr_t)act) & 15) return VK_BAD_ARGUMENT;
+    const int wide_tiles = vk_moe_max_tiles(pairs, experts, GT_TILE);
+    dim3 up(wide_tiles, (ff + 63) / 64), down(wide_tiles, (width + GT_TILE - 1) / GT_TILE);
+    if (up.y > 65535 || down.y > 65535) return VK_UNSUPPORTED_SIZE;
+    static bool sized = false;
+    if (!sized) {
+      hipError_t e1 = hipFuncSetAttribute((const void*)moe_gate_up_mma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES);
+      hipError_t e2 = hipFuncSetAttribute((const void*)moe_down_mma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS_BYTES);
+      if (e1 != hipSuccess || e2 != hipSuccess) return (int)(e1 != hipSuccess ? e1 : e2);
+      sized = true;
+    }
+    moe_gate_up_mma_kernel<<<up, 256, GT_LDS_BYTES, s>>>((const __bf16*)h, ldh, (const __bf16*)wg, (const __bf16*)wu,
+                                                        offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
+                                                        (__bf16*)act);
+    VK_LAUNCH_CHECK();
+    moe_down_mma_kernel<<<down, 256, GT_LDS_BYTES, s>>>((const __bf16*)act, (const __bf16*)wd, offsets, order, tiles,
+                                                        num_tiles, width, ff, pair_out);
+    VK_LAUNCH_CHECK();
+    const long long all = (long long)num_tokens * width;
+    moe_combine_kernel<<<(unsigned)((all + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, all, residual);
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+  const int max_tiles = vk_moe_max_tiles(pairs, experts, MOE_TILE);
   dim3 up_grid(max_tiles, (ff + MOE_TILE - 1) / MOE_TILE), down_grid(max_tiles, (width + MOE_TILE - 1) / MOE_TILE);
   if (up_grid.y > 65535 || down_grid.y > 65535) return VK_UNSUPPORTED_SIZE;
   if (dtype == DT_F32) {

@@ -5,10 +5,8 @@
 // that is used again needs no clearing.  The tokens of a step lie flat, entry after entry; `entry_start[e]` is
 // the first token of entry e, `entry_first_pos[e]` its position in the request, `slots[e]` the state row.
 //
-// The recurrence kernels give one lane a column of a head's state matrix (all key channels of one value
-// channel): the products with k, q and r are then sums inside a lane, in ascending key order, and do not
-// depend on what else is in the launch.  A wave owns 64 value channels of one (entry, head) and walks the
-// entry's tokens in order.
+// The recurrence kernels keep a head's state matrix in registers, a column of it spread over four lanes, and walk an
+// entry's tokens in order; a sum over the key channels has one fixed order, whatever else is in the launch.
 #include "common.h"
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
@@ -98,97 +96,165 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
+// The two recurrences share their shape.  A workgroup of four waves owns 64 value channels of one (entry, head); a
+// wave owns 16 of them, and its four groups of 16 lanes each a quarter of the key channels: a lane keeps R rows of
+// one column of the state in registers (4 R >= dim; rows past dim stay zero).  Sums over the key channels are R
+// terms in a lane, in ascending order, then two exchanges between the lane groups.  The entry's tokens are walked in
+// blocks of 16: a block's k, q (or r, k, decay), values and gates are fetched into registers while the block
+// before is worked on, and passed on through LDS, so that a token's step waits for no memory.
+constexpr int REC_BLOCK = 16;    // tokens per LDS block
+
+__device__ __forceinline__ float across_groups(float v) {
+  v += __shfl_xor(v, 16, WAVE);
+  v += __shfl_xor(v, 32, WAVE);
+  return v;
+}
+
 // Gated delta rule.  Per head, with S [dim, vdim]:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
-// Grid (entries, heads, ceil(vdim / 64)), one wave each.  Dynamic LDS: dim * 64 floats of state and 2 * dim of k, q.
-__global__ __launch_bounds__(64) void delta_rule_kernel(
+// Grid (entries, heads, ceil(vdim / 64)).  An LDS row of a token: [q: 4R | k: 4R | v: 64 | beta, decay].
+template <int R>
+__global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
     float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
     const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
     float* __restrict__ out) {
-  extern __shared__ float lds[];
-  float* S = lds;                    // [dim][64]
-  float* ks = lds + dim * WAVE;      // [dim]
-  float* qs = ks + dim;              // [dim]
-  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int v = blockIdx.z * WAVE + lane;
+  constexpr int DP = 4 * R, ROW = 2 * DP + 64 + 2, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  __shared__ float rows[COUNT];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane >> 4, d0 = grp * R;
+  const int v0 = blockIdx.z * 64, mine_col = wave * 16 + (lane & 15), v = v0 + mine_col;
   const bool live = v < vdim;
   const int kh = h / (heads / kv_heads);
   const int C = 2 * kv_heads * dim + heads * vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
   float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * vdim;
   const bool fresh = entry_first[e] == 0;
-  for (int d = 0; d < dim; ++d) S[d * WAVE + lane] = (live && !fresh) ? mine[(long long)d * vdim + v] : 0.f;
-  for (int t = start; t < end; ++t) {
-    const float* row = qkv + (long long)t * C;
+  float S[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) S[i] = (live && !fresh && d0 + i < dim) ? mine[(long long)(d0 + i) * vdim + v] : 0.f;
+  // what this thread fetches of a block: element x of the block is token x / ROW, column x % ROW
+  float held[LOADS];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int x = tid + i * 256, j = x / ROW, col = x % ROW, t = t0 + j;
+      float value = 0.f;
+      if (x < COUNT && t < end) {
+        if (col < DP) { if (col < dim) value = qkv[(long long)t * C + kh * dim + col]; }
+        else if (col < 2 * DP) { if (col - DP < dim) value = qkv[(long long)t * C + (kv_heads + kh) * dim + col - DP]; }
+        else if (col < 2 * DP + 64) { if (v0 + col - 2 * DP < vdim) value = qkv[(long long)t * C + 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP]; }
+        else if (col == 2 * DP + 64) value = beta[(long long)t * heads + h];
+        else value = decay[(long long)t * heads + h];
+      }
+      held[i] = value;
+    }
+  };
+  fetch(start);
+  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+    __syncthreads();     // the block before has been read
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      if (tid + i * 256 < COUNT) rows[tid + i * 256] = held[i];
     __syncthreads();
-    for (int d = lane; d < dim; d += WAVE) {
-      qs[d] = row[kh * dim + d];
-      ks[d] = row[(kv_heads + kh) * dim + d];
+    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    const int count = min(REC_BLOCK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float* row = rows + j * ROW;
+      const float b = row[2 * DP + 64], g = row[2 * DP + 65], val = row[2 * DP + mine_col];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        S[i] *= g;
+        dot = fmaf(S[i], row[DP + d0 + i], dot);
+      }
+      const float u = b * (val - across_groups(dot));
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        S[i] = fmaf(row[DP + d0 + i], u, S[i]);
+        o = fmaf(S[i], row[d0 + i], o);
+      }
+      o = across_groups(o);
+      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = o;
     }
-    __syncthreads();
-    const float g = decay[(long long)t * heads + h], b = beta[(long long)t * heads + h];
-    const float val = live ? row[2 * kv_heads * dim + h * vdim + v] : 0.f;
-    float dot = 0.f;
-    for (int d = 0; d < dim; ++d) {
-      const float s = g * S[d * WAVE + lane];
-      S[d * WAVE + lane] = s;
-      dot = fmaf(s, ks[d], dot);
-    }
-    const float u = b * (val - dot);
-    float o = 0.f;
-    for (int d = 0; d < dim; ++d) {
-      const float s = fmaf(ks[d], u, S[d * WAVE + lane]);
-      S[d * WAVE + lane] = s;
-      o = fmaf(s, qs[d], o);
-    }
-    if (live) out[((long long)t * heads + h) * vdim + v] = o;
   }
-  if (live)
-    for (int d = 0; d < dim; ++d) mine[(long long)d * vdim + v] = S[d * WAVE + lane];
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (d0 + i < dim) mine[(long long)(d0 + i) * vdim + v] = S[i];
+  }
 }
 
-// ---------------------------------------------------------------------------------------------
 // RWKV-style time mixing.  Per head, with S [dim, dim]:  o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T,
 // w = exp(-exp(wraw + w0)) per key channel.  r, k, v, wraw are 32-bit [T, heads * dim] with row strides of their own.
-// Grid (entries, heads, ceil(dim / 64)), one wave each.  Dynamic LDS: dim * 64 floats of state and 3 * dim floats.
-__global__ __launch_bounds__(64) void wkv_rule_kernel(
+// Grid (entries, heads, ceil(dim / 64)).  An LDS row of a token: [r: 4R | k: 4R | w: 4R | v: 64].
+template <int R>
+__global__ __launch_bounds__(256) void wkv_rule_kernel(
     const float* __restrict__ r, long long ldr, const float* __restrict__ k, long long ldk, const float* __restrict__ v,
     long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
     const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
     int heads, float* __restrict__ out) {
-  extern __shared__ float lds[];
-  float* S = lds;                    // [dim][64]
-  float* rs = lds + dim * WAVE;      // r[d]
-  float* ks = rs + dim;              // k[d]
-  float* ws = ks + dim;              // decay[d]
-  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * WAVE + lane;
-  const bool live = col < dim;
+  constexpr int DP = 4 * R, ROW = 3 * DP + 64, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  __shared__ float rows[COUNT];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane >> 4, d0 = grp * R;
+  const int v0 = blockIdx.z * 64, mine_col = wave * 16 + (lane & 15), col_v = v0 + mine_col;
+  const bool live = col_v < dim;
   const int start = entry_start[e], end = entry_start[e + 1];
   float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * dim;
   const bool fresh = entry_first[e] == 0;
-  for (int d = 0; d < dim; ++d) S[d * WAVE + lane] = (live && !fresh) ? mine[(long long)d * dim + col] : 0.f;
-  for (int t = start; t < end; ++t) {
-    __syncthreads();
-    for (int d = lane; d < dim; d += WAVE) {
-      rs[d] = r[(long long)t * ldr + h * dim + d];
-      ks[d] = k[(long long)t * ldk + h * dim + d];
-      ws[d] = expf(-expf(wraw[(long long)t * ldw + h * dim + d] + w0[h * dim + d]));
-    }
-    __syncthreads();
-    const float val = live ? v[(long long)t * ldv + h * dim + col] : 0.f;
-    float o = 0.f;
-    for (int d = 0; d < dim; ++d) {
-      const float kv = ks[d] * val;
-      const float s = S[d * WAVE + lane];
-      o = fmaf(fmaf(bonus[h * dim + d], kv, s), rs[d], o);
-      S[d * WAVE + lane] = fmaf(ws[d], s, kv);
-    }
-    if (live) out[((long long)t * heads + h) * dim + col] = o;
+  float S[R], U[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    S[i] = (live && !fresh && d0 + i < dim) ? mine[(long long)(d0 + i) * dim + col_v] : 0.f;
+    U[i] = d0 + i < dim ? bonus[h * dim + d0 + i] : 0.f;
   }
-  if (live)
-    for (int d = 0; d < dim; ++d) mine[(long long)d * dim + col] = S[d * WAVE + lane];
+  float held[LOADS];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int x = tid + i * 256, j = x / ROW, col = x % ROW, t = t0 + j;
+      float value = 0.f;
+      if (x < COUNT && t < end) {
+        if (col < DP) { if (col < dim) value = r[(long long)t * ldr + h * dim + col]; }
+        else if (col < 2 * DP) { if (col - DP < dim) value = k[(long long)t * ldk + h * dim + col - DP]; }
+        else if (col < 3 * DP) {
+          const int d = col - 2 * DP;
+          if (d < dim) value = expf(-expf(wraw[(long long)t * ldw + h * dim + d] + w0[h * dim + d]));
+        } else if (v0 + col - 3 * DP < dim) value = v[(long long)t * ldv + h * dim + v0 + col - 3 * DP];
+      }
+      held[i] = value;
+    }
+  };
+  fetch(start);
+  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      if (tid + i * 256 < COUNT) rows[tid + i * 256] = held[i];
+    __syncthreads();
+    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    const int count = min(REC_BLOCK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float* row = rows + j * ROW;
+      const float val = row[3 * DP + mine_col];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        const float kv = row[DP + d0 + i] * val;
+        o = fmaf(fmaf(U[i], kv, S[i]), row[d0 + i], o);
+        S[i] = fmaf(row[2 * DP + d0 + i], S[i], kv);
+      }
+      o = across_groups(o);
+      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = o;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (d0 + i < dim) mine[(long long)(d0 + i) * dim + col_v] = S[i];
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -294,12 +360,18 @@ extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* d
                              int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, void* stream) {
   if (num_entries <= 0) return 0;
   if (kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
-  const long long bytes = ((long long)dim * WAVE + 2LL * dim) * 4;
-  if (!fits_lds(bytes) || heads > 65535) return VK_UNSUPPORTED_SIZE;
-  dim3 grid(num_entries, heads, (vdim + WAVE - 1) / WAVE);
-  delta_rule_kernel<<<grid, WAVE, (size_t)bytes, (hipStream_t)stream>>>(qkv, beta, decay, state, state_stride,
-                                                                        entry_start, entry_first, slots, kv_heads, dim,
-                                                                        heads, vdim, out);
+  if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  dim3 grid(num_entries, heads, (vdim + 63) / 64);
+  hipStream_t s = (hipStream_t)stream;
+#define VK_DELTA(R)                                                                                               \
+  delta_rule_kernel<R><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
+                                            kv_heads, dim, heads, vdim, out)
+  if (dim <= 16) VK_DELTA(4);
+  else if (dim <= 32) VK_DELTA(8);
+  else if (dim <= 64) VK_DELTA(16);
+  else if (dim <= 128) VK_DELTA(32);
+  else VK_DELTA(64);
+#undef VK_DELTA
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -310,12 +382,18 @@ extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long l
                            int dim, int heads, float* out, int num_entries, void* stream) {
   if (num_entries <= 0) return 0;
   if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
-  const long long bytes = ((long long)dim * WAVE + 3LL * dim) * 4;
-  if (!fits_lds(bytes) || heads > 65535) return VK_UNSUPPORTED_SIZE;
-  dim3 grid(num_entries, heads, (dim + WAVE - 1) / WAVE);
-  wkv_rule_kernel<<<grid, WAVE, (size_t)bytes, (hipStream_t)stream>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus,
-                                                                      state, state_stride, entry_start, entry_first,
-                                                                      slots, dim, heads, out);
+  if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  dim3 grid(num_entries, heads, (dim + 63) / 64);
+  hipStream_t s = (hipStream_t)stream;
+#define VK_WKV(R)                                                                                                  \
+  wkv_rule_kernel<R><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,       \
+                                          entry_start, entry_first, slots, dim, heads, out)
+  if (dim <= 16) VK_WKV(4);
+  else if (dim <= 32) VK_WKV(8);
+  else if (dim <= 64) VK_WKV(16);
+  else if (dim <= 128) VK_WKV(32);
+  else VK_WKV(64);
+#undef VK_WKV
   VK_LAUNCH_CHECK();
   return 0;
 }

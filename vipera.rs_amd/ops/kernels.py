@@ -925,7 +925,7 @@ def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # --- recurrent mixers ---------------------------------------------------------------------------
-RECURRENT_MAX_KEY_DIM = 240    # a wave's 64 columns of a head's state and its k, q (r, decay) rows share 64 KB of LDS
+RECURRENT_MAX_KEY_DIM = 256    # a lane keeps a quarter of a state column's rows in registers: at most 64
 
 
 def _entries_ok(batch_arrays, num_entries: int) -> None:
@@ -1109,15 +1109,18 @@ def head_linear(a: torch.Tensor, a_head_stride: int, k: int, w: torch.Tensor, ou
 
 
 # --- mixture of experts ---------------------------------------------------------------------------
-MOE_TILE = 64
+def moe_tile_rows(h: torch.Tensor, width: int, ff: int) -> int:
+    """Places per tile of the experts' products for activations ``h``: 128 on the matrix cores (bfloat16, widths that
+    are multiples of 8), 64 as 32-bit FMAs.  The grouping has to be made for the same number."""
+    return 128 if (h.dtype == torch.bfloat16 and width % 8 == 0 and ff % 8 == 0 and h.stride(0) % 8 == 0) else 64
 
 
-def moe_max_tiles(pairs: int, experts: int) -> int:
-    return (pairs + MOE_TILE - 1) // MOE_TILE + experts
+def moe_max_tiles(pairs: int, experts: int, tile_rows: int = 64) -> int:
+    return (pairs + tile_rows - 1) // tile_rows + experts
 
 
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, offsets: torch.Tensor,
-              order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor) -> None:
+              order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, tile_rows: int = 64) -> None:
     """Each token's ``top`` largest router logits (lowest id first among equals) with the softmax over those, and the
     (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``."""
     _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
@@ -1127,10 +1130,10 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
     _i32(ids, offsets, order, tiles, num_tiles)
     _f32(weights, "moe_route: weights")
     _need(ids.numel() == tokens * top and weights.numel() == tokens * top and order.numel() == tokens * top
-          and offsets.numel() == experts + 1 and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts)
-          and num_tiles.numel() == 1, "moe_route: output sizes")
-    fn = _fn("moe", "vk_moe_route", [_p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
-    _status(fn(_ptr(logits), experts, top, tokens, _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles),
+          and offsets.numel() == experts + 1 and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts, tile_rows)
+          and num_tiles.numel() == 1 and tile_rows in (64, 128), "moe_route: output sizes")
+    fn = _fn("moe", "vk_moe_route", [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
+    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles),
                _ptr(num_tiles), _stream()), "moe_route")
 
 
@@ -1154,7 +1157,8 @@ def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_dow
           "moe_experts: output shapes")
     _i32(offsets, order, tiles, num_tiles)
     _need(offsets.numel() == experts + 1 and order.numel() == tokens * top
-          and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts), "moe_experts: grouping")
+          and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts, moe_tile_rows(h, width, ff)),
+          "moe_experts: grouping (made by moe_route with moe_tile_rows(h, width, ff))")
     fn = _fn("moe", "vk_moe_experts", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p, _p, _p])
     _status(fn(_ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _dt(h, "h"), _ptr(offsets), _ptr(order),
                _ptr(tiles), _ptr(num_tiles), _ptr(weights), tokens, experts, top, width, ff, float(limit), float(alpha),

@@ -70,14 +70,15 @@ class MixtureOfExperts(FeedForward):
         pairs = tokens * self.top
         logits = torch.empty((tokens, self.experts), dtype=torch.float32, device=device)
         linear(h, self.w_router, None, logits)
-        ints = torch.empty(2 * pairs + self.experts + 2 + 2 * kernels.moe_max_tiles(pairs, self.experts),
+        tile_rows = kernels.moe_tile_rows(h, self.hidden, self.inter)
+        ints = torch.empty(2 * pairs + self.experts + 2 + 2 * kernels.moe_max_tiles(pairs, self.experts, tile_rows),
                            dtype=torch.int32, device=device)
         ids, order = ints[:pairs], ints[pairs:2 * pairs]
         offsets = ints[2 * pairs:2 * pairs + self.experts + 1]
         num_tiles = ints[2 * pairs + self.experts + 1:2 * pairs + self.experts + 2]
         tiles = ints[2 * pairs + self.experts + 2:]
         weights = torch.empty(pairs, dtype=torch.float32, device=device)
-        kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles)
+        kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles, tile_rows)
         act = self.runtime.empty((pairs, self.inter))
         pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
         kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,
