@@ -31,8 +31,9 @@ def test_a_shared_cache_keeps_the_widest_window_of_its_readers():
     assert second["shares_cache"] and not first["shares_cache"]
     needs = declare_cache_needs(cfg)
     assert needs[3].owner == 0 and needs[0].kv == needs[3].kv and needs[0].kv.window == 29 and needs[0].kv.head_dim == 64
-    assert needs[1].kv is None and needs[1].state.shape == (3 * 16 * 16 + 96,)
-    assert needs[2].state.shape == (4 * 16 * 24 + 3 * (2 * 2 * 16 + 4 * 24),)
+    assert needs[1].kv is None and needs[1].state.shape == (3 * 256 + 96,)     # a head's 16 x 16 matrix, then the last h
+    # heads of 16 x 24 padded to two value tiles of 16, then three rows of the convolution's inputs
+    assert needs[2].state.shape == (4 * 2 * 256 + 3 * (2 * 2 * 16 + 4 * 24),)
     # one reader without a window: everything is kept
     other = config_from_dict(G.written_config(G.G2))
     assert [s.mixer.params.get("retain") for s in other.layer_specs() if s.mixer.kind == "latent_attention"] == [0, 0]

@@ -96,42 +96,55 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
-// The two recurrences share their shape.  A workgroup of four waves owns 64 value channels of one (entry, head); a
-// wave owns 16 of them, and its four groups of 16 lanes each a quarter of the key channels: a lane keeps R rows of
-// one column of the state in registers (4 R >= dim; rows past dim stay zero).  Sums over the key channels are R
-// terms in a lane, in ascending order, then two exchanges between the lane groups.  The entry's tokens are walked in
-// blocks of 16: a block's k, q (or r, k, decay), values and gates are fetched into registers while the block
-// before is worked on, and passed on through LDS, so that a token's step waits for no memory.
+// The two recurrences share their shape.  A workgroup of four waves owns 16 value channels of one (entry, head), a
+// wave four of them; the sixteen lanes of a row of the wave share one value channel and each keeps R of its key
+// channels in registers (16 R >= dim; rows past dim stay zero).  A sum over the key channels is R terms in a lane, in
+// ascending order, then four exchanges inside the 16-lane row (DPP, no LDS).  The entry's tokens are walked in
+// blocks of 16: a block's k, q (or r, k, decay), values and gates are fetched into registers while the block before
+// is worked on, and passed on through LDS, so that a token's step waits for no memory.
+//
+// The state of a head lies in memory as the kernel holds it: [value tile of 16][thread of 256][R], so that a
+// lane's R numbers are contiguous and a workgroup reads and writes one contiguous run.  Nobody else reads it.
 constexpr int REC_BLOCK = 16;    // tokens per LDS block
+constexpr int REC_COLS = 16;     // value channels per workgroup
 
-__device__ __forceinline__ float across_groups(float v) {
-  v += __shfl_xor(v, 16, WAVE);
-  v += __shfl_xor(v, 32, WAVE);
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
+  return v + __int_as_float(moved);
+}
+
+// The sum over the 16 lanes of a row, in every lane: neighbours, pairs of neighbours, the halves of eight, the eights.
+__device__ __forceinline__ float row_sum16(float v) {
+  v = dpp_add<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  v = dpp_add<0x141>(v);    // row_half_mirror: the other quad of the eight
+  v = dpp_add<0x140>(v);    // row_mirror: the other eight
   return v;
 }
 
 // Gated delta rule.  Per head, with S [dim, vdim]:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
-// Grid (entries, heads, ceil(vdim / 64)).  An LDS row of a token: [q: 4R | k: 4R | v: 64 | beta, decay].
+// Grid (entries, heads, ceil(vdim / 16)).  An LDS row of a token: [q: 16R | k: 16R | v: 16 | beta, decay].
 template <int R>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
     float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
     const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
     float* __restrict__ out) {
-  constexpr int DP = 4 * R, ROW = 2 * DP + 64 + 2, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  constexpr int DP = 16 * R, ROW = 2 * DP + REC_COLS + 2, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int grp = lane >> 4, d0 = grp * R;
-  const int v0 = blockIdx.z * 64, mine_col = wave * 16 + (lane & 15), v = v0 + mine_col;
+  const int grp = lane & 15, d0 = grp * R;
+  const int v0 = blockIdx.z * REC_COLS, mine_col = wave * 4 + (lane >> 4), v = v0 + mine_col;
   const bool live = v < vdim;
   const int kh = h / (heads / kv_heads);
   const int C = 2 * kv_heads * dim + heads * vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
-  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * vdim;
+  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z + blockIdx.z) * 256 + tid) * R;
   const bool fresh = entry_first[e] == 0;
   float S[R];
 #pragma unroll
-  for (int i = 0; i < R; ++i) S[i] = (live && !fresh && d0 + i < dim) ? mine[(long long)(d0 + i) * vdim + v] : 0.f;
+  for (int i = 0; i < R; ++i) S[i] = fresh ? 0.f : mine[i];
   // what this thread fetches of a block: element x of the block is token x / ROW, column x % ROW
   float held[LOADS];
   auto fetch = [&](int t0) {
@@ -142,8 +155,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
       if (x < COUNT && t < end) {
         if (col < DP) { if (col < dim) value = qkv[(long long)t * C + kh * dim + col]; }
         else if (col < 2 * DP) { if (col - DP < dim) value = qkv[(long long)t * C + (kv_heads + kh) * dim + col - DP]; }
-        else if (col < 2 * DP + 64) { if (v0 + col - 2 * DP < vdim) value = qkv[(long long)t * C + 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP]; }
-        else if (col == 2 * DP + 64) value = beta[(long long)t * heads + h];
+        else if (col < 2 * DP + REC_COLS) { if (v0 + col - 2 * DP < vdim) value = qkv[(long long)t * C + 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP]; }
+        else if (col == 2 * DP + REC_COLS) value = beta[(long long)t * heads + h];
         else value = decay[(long long)t * heads + h];
       }
       held[i] = value;
@@ -160,34 +173,37 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     const int count = min(REC_BLOCK, end - t0);
     for (int j = 0; j < count; ++j) {
       const float* row = rows + j * ROW;
-      const float b = row[2 * DP + 64], g = row[2 * DP + 65], val = row[2 * DP + mine_col];
+      const float b = row[2 * DP + REC_COLS], g = row[2 * DP + REC_COLS + 1], val = row[2 * DP + mine_col];
+      float kk[R], qq[R];
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        kk[i] = row[DP + d0 + i];
+        qq[i] = row[d0 + i];
+      }
       float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
         S[i] *= g;
-        dot = fmaf(S[i], row[DP + d0 + i], dot);
+        dot = fmaf(S[i], kk[i], dot);
       }
-      const float u = b * (val - across_groups(dot));
+      const float u = b * (val - row_sum16(dot));
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        S[i] = fmaf(row[DP + d0 + i], u, S[i]);
-        o = fmaf(S[i], row[d0 + i], o);
+        S[i] = fmaf(kk[i], u, S[i]);
+        o = fmaf(S[i], qq[i], o);
       }
-      o = across_groups(o);
+      o = row_sum16(o);
       if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = o;
     }
   }
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-      if (d0 + i < dim) mine[(long long)(d0 + i) * vdim + v] = S[i];
-  }
+  for (int i = 0; i < R; ++i) mine[i] = S[i];
 }
 
 // RWKV-style time mixing.  Per head, with S [dim, dim]:  o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T,
 // w = exp(-exp(wraw + w0)) per key channel.  r, k, v, wraw are 32-bit [T, heads * dim] with row strides of their own.
-// Grid (entries, heads, ceil(dim / 64)).  An LDS row of a token: [r: 4R | k: 4R | w: 4R | v: 64].
+// Grid (entries, heads, ceil(dim / 16)).  An LDS row of a token: [r: 16R | k: 16R | w: 16R | v: 16].
 template <int R>
 __global__ __launch_bounds__(256) void wkv_rule_kernel(
     const float* __restrict__ r, long long ldr, const float* __restrict__ k, long long ldk, const float* __restrict__ v,
@@ -195,19 +211,19 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
     const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
     int heads, float* __restrict__ out) {
-  constexpr int DP = 4 * R, ROW = 3 * DP + 64, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  constexpr int DP = 16 * R, ROW = 3 * DP + REC_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int grp = lane >> 4, d0 = grp * R;
-  const int v0 = blockIdx.z * 64, mine_col = wave * 16 + (lane & 15), col_v = v0 + mine_col;
+  const int grp = lane & 15, d0 = grp * R;
+  const int v0 = blockIdx.z * REC_COLS, mine_col = wave * 4 + (lane >> 4), col_v = v0 + mine_col;
   const bool live = col_v < dim;
   const int start = entry_start[e], end = entry_start[e + 1];
-  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * dim) * dim;
+  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z + blockIdx.z) * 256 + tid) * R;
   const bool fresh = entry_first[e] == 0;
   float S[R], U[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    S[i] = (live && !fresh && d0 + i < dim) ? mine[(long long)(d0 + i) * dim + col_v] : 0.f;
+    S[i] = fresh ? 0.f : mine[i];
     U[i] = d0 + i < dim ? bonus[h * dim + d0 + i] : 0.f;
   }
   float held[LOADS];
@@ -246,15 +262,12 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
         o = fmaf(fmaf(U[i], kv, S[i]), row[d0 + i], o);
         S[i] = fmaf(row[2 * DP + d0 + i], S[i], kv);
       }
-      o = across_groups(o);
+      o = row_sum16(o);
       if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = o;
     }
   }
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < R; ++i)
-      if (d0 + i < dim) mine[(long long)(d0 + i) * dim + col_v] = S[i];
-  }
+  for (int i = 0; i < R; ++i) mine[i] = S[i];
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -355,22 +368,28 @@ extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* c
   return 0;
 }
 
+// Floats of one head's state as the recurrence kernels lay it out: value tiles of 16 x 256 threads x R.
+extern "C" long long vk_recurrent_head_floats(int dim, int vdim) {
+  const int r = dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16;
+  return (long long)((vdim + REC_COLS - 1) / REC_COLS) * 256 * r;
+}
+
 extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
                              long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
                              int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, void* stream) {
   if (num_entries <= 0) return 0;
   if (kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
-  dim3 grid(num_entries, heads, (vdim + 63) / 64);
+  dim3 grid(num_entries, heads, (vdim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
 #define VK_DELTA(R)                                                                                               \
   delta_rule_kernel<R><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
                                             kv_heads, dim, heads, vdim, out)
-  if (dim <= 16) VK_DELTA(4);
-  else if (dim <= 32) VK_DELTA(8);
-  else if (dim <= 64) VK_DELTA(16);
-  else if (dim <= 128) VK_DELTA(32);
-  else VK_DELTA(64);
+  if (dim <= 16) VK_DELTA(1);
+  else if (dim <= 32) VK_DELTA(2);
+  else if (dim <= 64) VK_DELTA(4);
+  else if (dim <= 128) VK_DELTA(8);
+  else VK_DELTA(16);
 #undef VK_DELTA
   VK_LAUNCH_CHECK();
   return 0;
@@ -383,16 +402,16 @@ extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long l
   if (num_entries <= 0) return 0;
   if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
-  dim3 grid(num_entries, heads, (dim + 63) / 64);
+  dim3 grid(num_entries, heads, (dim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
 #define VK_WKV(R)                                                                                                  \
   wkv_rule_kernel<R><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,       \
                                           entry_start, entry_first, slots, dim, heads, out)
-  if (dim <= 16) VK_WKV(4);
-  else if (dim <= 32) VK_WKV(8);
-  else if (dim <= 64) VK_WKV(16);
-  else if (dim <= 128) VK_WKV(32);
-  else VK_WKV(64);
+  if (dim <= 16) VK_WKV(1);
+  else if (dim <= 32) VK_WKV(2);
+  else if (dim <= 64) VK_WKV(4);
+  else if (dim <= 128) VK_WKV(8);
+  else VK_WKV(16);
 #undef VK_WKV
   VK_LAUNCH_CHECK();
   return 0;

@@ -928,6 +928,13 @@ def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
 RECURRENT_MAX_KEY_DIM = 256    # a lane keeps a quarter of a state column's rows in registers: at most 64
 
 
+def recurrent_head_floats(dim: int, vdim: int) -> int:
+    """Floats of one head's ``[dim, vdim]`` state as the recurrence kernels keep it in a slot: padded to value tiles of
+    16 and to 16, 32, 64, 128 or 256 key channels, in the order of the kernel's threads."""
+    rows = 1 if dim <= 16 else 2 if dim <= 32 else 4 if dim <= 64 else 8 if dim <= 128 else 16
+    return (vdim + 15) // 16 * 256 * rows
+
+
 def _entries_ok(batch_arrays, num_entries: int) -> None:
     entry_start, entry_first, slots = batch_arrays
     _i32(entry_start, entry_first, slots)
@@ -972,7 +979,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
                entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, kv_heads: int, dim: int,
                heads: int, vdim: int, out: torch.Tensor, num_entries: int) -> None:
     """The gated delta rule over every entry's tokens in order, from and into the entries' state rows (the first
-    ``heads * dim * vdim`` floats of a row, ``[heads, dim, vdim]``); ``out`` 32-bit ``[tokens, heads * vdim]``."""
+    ``heads * recurrent_head_floats(dim, vdim)`` floats of a row, in the kernel's own order); ``out`` 32-bit ``[tokens, heads * vdim]``."""
     _dev(qkv, beta, decay, state, entry_start, entry_first, slots, out)
     tokens = qkv.shape[0]
     channels = 2 * kv_heads * dim + heads * vdim
@@ -981,7 +988,7 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
     for t in (qkv, beta, decay, out):
         _f32(t, "delta_rule: operands")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
-          and state.shape[1] >= heads * dim * vdim, "delta_rule: state row")
+          and state.shape[1] >= heads * recurrent_head_floats(dim, vdim), "delta_rule: state row")
     _entries_ok((entry_start, entry_first, slots), num_entries)
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"delta_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
@@ -995,7 +1002,8 @@ def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tens
              slots: torch.Tensor, dim: int, heads: int, out: torch.Tensor, num_entries: int) -> None:
     """RWKV-style time mixing over every entry's tokens in order: ``o = (S + diag(u) k v^T)^T r``, then
     ``S = diag(w) S + k v^T`` with ``w = exp(-exp(wraw + w0))``.  ``r, k, v, wraw``: 32-bit ``[tokens, heads * dim]``
-    (row-strided views are fine); state rows start with ``[heads, dim, dim]``."""
+    (row-strided views are fine); state rows start with the heads' matrices
+    (``heads * recurrent_head_floats(dim, dim)`` floats, in the kernel's own order)."""
     _dev(r, k, v, wraw, w0, bonus, state, entry_start, entry_first, slots, out)
     tokens, width = out.shape[0], heads * dim
     for name, t in (("r", r), ("k", k), ("v", v), ("wraw", wraw)):
@@ -1005,7 +1013,7 @@ def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tens
     _f32(out, "wkv_rule: out")
     _need(out.shape == (tokens, width), "wkv_rule: out shape")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
-          and state.shape[1] >= heads * dim * dim, "wkv_rule: state row")
+          and state.shape[1] >= heads * recurrent_head_floats(dim, dim), "wkv_rule: state row")
     _entries_ok((entry_start, entry_first, slots), num_entries)
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"wkv_rule: a head width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")

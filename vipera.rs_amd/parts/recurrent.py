@@ -72,7 +72,7 @@ class GatedDelta(Mixer):
     def declare_cache(cls, spec: PartSpec):
         p = spec.params
         _, _, channels = cls._sizes(p)
-        floats = int(p["heads"]) * int(p["dim"]) * int(p["vdim"]) + (int(p["conv"]) - 1) * channels
+        floats = int(p["heads"]) * kernels.recurrent_head_floats(int(p["dim"]), int(p["vdim"])) + (int(p["conv"]) - 1) * channels
         return None, StateSpec((floats,), torch.float32)
 
     @classmethod
@@ -105,7 +105,7 @@ class GatedDelta(Mixer):
         beta, decay = torch.empty((tokens, self.heads), **f32), torch.empty((tokens, self.heads), **f32)
         g_col = self.channels
         b_col = g_col + self.vw
-        matrices = self.heads * self.dim * self.vdim
+        matrices = self.heads * kernels.recurrent_head_floats(self.dim, self.vdim)
         kernels.delta_prepare(proj, self.conv, state, matrices, batch.entry_of_token, batch.entry_start,
                               batch.entry_first_pos, batch.slots, self.a_log, self.dt_bias, self.kv_heads, self.dim,
                               self.heads, self.vdim, b_col, b_col + self.heads, UNIT_EPS, qkv, beta, decay, entries)
@@ -148,7 +148,8 @@ class Wkv(Mixer):
     @classmethod
     def declare_cache(cls, spec: PartSpec):
         p = spec.params
-        return None, StateSpec((int(p["heads"]) * int(p["dim"]) ** 2 + int(p["hidden"]),), torch.float32)
+        matrices = int(p["heads"]) * kernels.recurrent_head_floats(int(p["dim"]), int(p["dim"]))
+        return None, StateSpec((matrices + int(p["hidden"]),), torch.float32)
 
     @classmethod
     def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
@@ -171,7 +172,7 @@ class Wkv(Mixer):
         tokens, entries = residual.shape[0], batch.num_entries
         device = residual.device
         f32 = dict(dtype=torch.float32, device=device)
-        matrices = self.heads * self.dim * self.dim
+        matrices = self.heads * kernels.recurrent_head_floats(self.dim, self.dim)
         mixes = self.runtime.empty((len(self.MIXES), tokens, self.hidden))
         kernels.token_shift(h, self.mu, state, matrices, batch.entry_of_token, batch.entry_start,
                             batch.entry_first_pos, batch.slots, mixes, entries)
