@@ -23,6 +23,8 @@ constexpr int GT_LDS_BYTES = 2 * GT_STAGE;
 // a_row(r): pointer to activation row r of the tile (r < 128) or nullptr; w_row(r): pointer to weight row r of the
 // tile or nullptr.  After the call acc[tn][tm] holds, for this lane, weight rows wn * 64 + tn * 16 + (lane / 16) * 4
 // + 0..3 of activation row wm * 64 + tm * 16 + lane % 16.
+// Chunks that do not exist are not loaded (measured against reading them at a fixed address and masking: a tile of a
+// decode step, which is mostly empty rows, took 40 % longer that way).
 template <typename ARow, typename WRow>
 __device__ __forceinline__ void group_tile_mma(ARow a_row, WRow w_row, int K, unsigned char* lds,
                                                gt_f32x4 (&acc)[4][4]) {

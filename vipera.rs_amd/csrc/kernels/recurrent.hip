@@ -151,14 +151,18 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int x = tid + i * 256, j = x / ROW, col = x % ROW, t = t0 + j;
-      float value = 0.f;
-      if (x < COUNT && t < end) {
-        if (col < DP) { if (col < dim) value = qkv[(long long)t * C + kh * dim + col]; }
-        else if (col < 2 * DP) { if (col - DP < dim) value = qkv[(long long)t * C + (kv_heads + kh) * dim + col - DP]; }
-        else if (col < 2 * DP + REC_COLS) { if (v0 + col - 2 * DP < vdim) value = qkv[(long long)t * C + 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP]; }
-        else if (col == 2 * DP + REC_COLS) value = beta[(long long)t * heads + h];
-        else value = decay[(long long)t * heads + h];
-      }
+      // one load per element and no branch around it (a load inside a branch would be waited for there, and a
+      // block's loads would arrive one after the other): the address is chosen by selects, a clamped one where
+      // the element does not exist, and the value is masked afterwards
+      const bool is_q = col < DP, is_k = !is_q && col < 2 * DP, is_v = !is_q && !is_k && col < 2 * DP + REC_COLS;
+      const bool is_b = col == 2 * DP + REC_COLS;
+      const int d = is_q ? col : col - DP, c = col - 2 * DP;
+      const bool ok = x < COUNT && t < end && (is_q || is_k ? d < dim : is_v ? v0 + c < vdim : true);
+      const long long tt = ok ? t : start;
+      const float* base = (is_q || is_k || is_v) ? qkv + tt * C : (is_b ? beta : decay) + tt * heads + h;
+      const int within = is_q ? kh * dim + d : is_k ? (kv_heads + kh) * dim + d : is_v ? 2 * kv_heads * dim + h * vdim + v0 + c : 0;
+      const float loaded = base[ok ? within : 0];
+      const float value = ok ? loaded : 0.f;
       held[i] = value;
     }
   };
@@ -171,30 +175,42 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     __syncthreads();
     if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
     const int count = min(REC_BLOCK, end - t0);
-    for (int j = 0; j < count; ++j) {
+    // a token's numbers are read from LDS while the token before it is worked on
+    float kk[R], qq[R], b, g, val;
+    auto read = [&](int j) {
       const float* row = rows + j * ROW;
-      const float b = row[2 * DP + REC_COLS], g = row[2 * DP + REC_COLS + 1], val = row[2 * DP + mine_col];
-      float kk[R], qq[R];
+      b = row[2 * DP + REC_COLS], g = row[2 * DP + REC_COLS + 1], val = row[2 * DP + mine_col];
 #pragma unroll
       for (int i = 0; i < R; ++i) {
         kk[i] = row[DP + d0 + i];
         qq[i] = row[d0 + i];
       }
-      float dot = 0.f;
+    };
+    read(0);
+    for (int j = 0; j < count; ++j) {
+      float k_now[R], q_now[R];
+      const float b_now = b, g_now = g, val_now = val;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        S[i] *= g;
-        dot = fmaf(S[i], kk[i], dot);
+        k_now[i] = kk[i];
+        q_now[i] = qq[i];
       }
-      const float u = b * (val - row_sum16(dot));
-      float o = 0.f;
+      if (j + 1 < count) read(j + 1);
+      float dot[2] = {0.f, 0.f};     // two chains, even and odd rows, added at the end: a fixed order
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        S[i] = fmaf(kk[i], u, S[i]);
-        o = fmaf(S[i], qq[i], o);
+        S[i] *= g_now;
+        dot[i & 1] = fmaf(S[i], k_now[i], dot[i & 1]);
       }
-      o = row_sum16(o);
-      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = o;
+      const float u = b_now * (val_now - row_sum16(dot[0] + dot[1]));
+      float o[2] = {0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        S[i] = fmaf(k_now[i], u, S[i]);
+        o[i & 1] = fmaf(S[i], q_now[i], o[i & 1]);
+      }
+      const float sum = row_sum16(o[0] + o[1]);
+      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = sum;
     }
   }
 #pragma unroll
@@ -231,15 +247,16 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int x = tid + i * 256, j = x / ROW, col = x % ROW, t = t0 + j;
-      float value = 0.f;
-      if (x < COUNT && t < end) {
-        if (col < DP) { if (col < dim) value = r[(long long)t * ldr + h * dim + col]; }
-        else if (col < 2 * DP) { if (col - DP < dim) value = k[(long long)t * ldk + h * dim + col - DP]; }
-        else if (col < 3 * DP) {
-          const int d = col - 2 * DP;
-          if (d < dim) value = expf(-expf(wraw[(long long)t * ldw + h * dim + d] + w0[h * dim + d]));
-        } else if (v0 + col - 3 * DP < dim) value = v[(long long)t * ldv + h * dim + v0 + col - 3 * DP];
-      }
+      // branch-free, as in the delta rule's kernel: selected addresses, one load each, masked values
+      const bool is_r = col < DP, is_k = !is_r && col < 2 * DP, is_w = !is_r && !is_k && col < 3 * DP;
+      const int d = is_r ? col : is_k ? col - DP : col - 2 * DP, c = col - 3 * DP;
+      const bool ok = x < COUNT && t < end && (is_r || is_k || is_w ? d < dim : v0 + c < dim);
+      const long long tt = ok ? t : start;
+      const float* base = is_r ? r + tt * ldr : is_k ? k + tt * ldk : is_w ? wraw + tt * ldw : v + tt * ldv;
+      const int within = ok ? h * dim + ((is_r || is_k || is_w) ? d : v0 + c) : 0;
+      const float loaded = base[within];
+      const float shift = w0[(ok && is_w) ? h * dim + d : 0];
+      const float value = !ok ? 0.f : is_w ? expf(-expf(loaded + shift)) : loaded;
       held[i] = value;
     }
   };
@@ -252,18 +269,37 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
     __syncthreads();
     if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
     const int count = min(REC_BLOCK, end - t0);
-    for (int j = 0; j < count; ++j) {
+    float rr[R], kk[R], ww[R], val;
+    auto read = [&](int j) {
       const float* row = rows + j * ROW;
-      const float val = row[3 * DP + mine_col];
-      float o = 0.f;
+      val = row[3 * DP + mine_col];
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        const float kv = row[DP + d0 + i] * val;
-        o = fmaf(fmaf(U[i], kv, S[i]), row[d0 + i], o);
-        S[i] = fmaf(row[2 * DP + d0 + i], S[i], kv);
+        rr[i] = row[d0 + i];
+        kk[i] = row[DP + d0 + i];
+        ww[i] = row[2 * DP + d0 + i];
       }
-      o = row_sum16(o);
-      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = o;
+    };
+    read(0);
+    for (int j = 0; j < count; ++j) {
+      float r_now[R], k_now[R], w_now[R];
+      const float val_now = val;
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        r_now[i] = rr[i];
+        k_now[i] = kk[i];
+        w_now[i] = ww[i];
+      }
+      if (j + 1 < count) read(j + 1);
+      float o[2] = {0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < R; ++i) {
+        const float kv = k_now[i] * val_now;
+        o[i & 1] = fmaf(fmaf(U[i], kv, S[i]), r_now[i], o[i & 1]);
+        S[i] = fmaf(w_now[i], S[i], kv);
+      }
+      const float sum = row_sum16(o[0] + o[1]);
+      if (live && grp == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = sum;
     }
   }
 #pragma unroll
