@@ -15,13 +15,9 @@ constexpr int MOE_TILE = 64;      // places per tile of the 32-bit products; the
 // ---------------------------------------------------------------------------------------------
 // One wave per token: the `top` largest of E logits (the lowest id wins a tie), and the softmax over those.
 // Lane l looks after experts l, l + 64, ...; a bit per expert of its own says which are taken (E <= 4096).
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
-                                                        int num_tokens, int* __restrict__ ids,
-                                                        float* __restrict__ weights) {
+__device__ __forceinline__ void route_token(const float* __restrict__ logits, int experts, int top, int t, int lane,
+                                            int* __restrict__ ids, float* __restrict__ weights) {
   constexpr int NONE = 0x7fffffff;
-  const int lane = threadIdx.x & (WAVE - 1);
-  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  if (t >= num_tokens) return;
   const float* z = logits + (long long)t * experts;
   unsigned long long taken = 0;
   float first = 0.f, sum = 0.f, mine = 0.f;      // lane j keeps the weight of choice j
@@ -54,15 +50,31 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   if (lane < top) weights[(long long)t * top + lane] = mine / sum;
 }
 
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
+                                                        int num_tokens, int* __restrict__ ids,
+                                                        float* __restrict__ weights) {
+  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (t < num_tokens) route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights);
+}
+
 // One workgroup: counts per expert, offsets, the pairs' places, and the list of tiles.
 //   offsets [E + 1], order [P], tiles [max_tiles][2] = (expert, first place), num_tiles [1]
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, int pairs, int experts,
-                                                         int tile_rows, int* __restrict__ offsets,
+// With `logits`: the same workgroup routes the step's tokens first, a wave per token in turn (a step of few tokens:
+// one launch instead of two).
+__global__ __launch_bounds__(1024) void moe_group_kernel(const float* __restrict__ logits, int top, int num_tokens,
+                                                         float* __restrict__ weights, int* __restrict__ ids, int pairs,
+                                                         int experts, int tile_rows, int* __restrict__ offsets,
                                                          int* __restrict__ order, int* __restrict__ tiles,
                                                          int* __restrict__ num_tiles) {
   extern __shared__ int shared[];      // counts [E], cursor [E]
   int* counts = shared;
   int* cursor = shared + experts;
+  if (logits) {
+    for (int t = threadIdx.x / WAVE; t < num_tokens; t += blockDim.x / WAVE)
+      route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights);
+    __threadfence_block();
+    __syncthreads();
+  }
   for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&counts[ids[p]], 1);
@@ -321,12 +333,16 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-  moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights);
-  VK_LAUNCH_CHECK();
   const long long pairs = (long long)num_tokens * top;
   if (pairs > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
-  moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(ids, (int)pairs, experts, tile_rows, offsets,
-                                                                       order, tiles, num_tiles);
+  const bool together = num_tokens <= 64;     // sixteen waves route four tokens each at most
+  if (!together) {
+    moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights);
+    VK_LAUNCH_CHECK();
+  }
+  moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(together ? logits : nullptr, top, num_tokens,
+                                                                       weights, ids, (int)pairs, experts, tile_rows,
+                                                                       offsets, order, tiles, num_tiles);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -20,78 +20,92 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : lo
 //   state row: `(taps - 1) * C` floats from `conv_offset` on, the inputs of the last taps - 1 tokens, oldest first
 //   ba    columns `b_col + h` and `a_col + h` of proj hold the projections for beta and the decay's step
 // Outputs (32-bit): qkv [T, C] (q unit * dim^-1/2, k unit, v), beta [T, heads], decay [T, heads].
-// One workgroup per token.
+// Grid (tokens, segments): a segment is one q or k head (its unit norm needs the whole head) or up to 1,024 value
+// channels.  No load sits behind a branch: where an input comes from (the step, the state, nowhere) picks an
+// address, and the value is masked.
+constexpr int PREP_SPAN = 1024;
+
+__device__ __forceinline__ float conv_input(const float* __restrict__ proj, long long ldp, const float* __restrict__ old,
+                                            int C, int taps, int t, int offset, bool fresh, int back, int c) {
+  const bool in_step = back <= offset, in_state = !in_step && !fresh;
+  const float* from = in_step ? proj + (long long)(t - back) * ldp + c
+                              : in_state ? old + (long long)(taps - 1 - (back - offset)) * C + c : proj + (long long)t * ldp + c;
+  const float x = *from;
+  return (in_step || in_state) ? x : 0.f;
+}
+
 __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const float* __restrict__ proj, long long ldp, const float* __restrict__ conv, int taps,
     const float* __restrict__ state, long long state_stride, long long conv_offset, const int* __restrict__ entry_of,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, int kv_heads, int dim, int heads, int vdim,
     int b_col, int a_col, float unit_eps, float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
-  extern __shared__ float row[];   // C floats
-  const int t = blockIdx.x;
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, seg = blockIdx.y;
   const int e = entry_of[t];
-  const int start = entry_start[e];
-  const int offset = t - start;
+  const int offset = t - entry_start[e];
   const bool fresh = entry_first[e] == 0;
-  const int C = 2 * kv_heads * dim + heads * vdim;
-  const float* old = state + (long long)slots[e] * state_stride + conv_offset;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float sum = 0.f;
-    for (int j = 0; j < taps; ++j) {
-      const int back = taps - 1 - j;            // how many tokens before this one
-      float x;
-      if (back <= offset) {
-        x = proj[(long long)(t - back) * ldp + c];
-      } else if (fresh) {
-        x = 0.f;
-      } else {
-        x = old[(long long)(taps - 1 - (back - offset)) * C + c];   // back - offset tokens before the entry
-      }
-      sum = fmaf(conv[(long long)c * taps + j], x, sum);
-    }
-    row[c] = silu_f(sum);
-  }
-  __syncthreads();
-  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
-  float* out = qkv + (long long)t * C;
   const int unit_heads = 2 * kv_heads;
-  for (int h = wave; h < unit_heads; h += waves) {
-    const float* src = row + h * dim;
-    float ss = 0.f;
-    for (int d = lane; d < dim; d += WAVE) ss += src[d] * src[d];
-    ss = wave_sum(ss);
-    float inv = 1.0f / sqrtf(ss + unit_eps);
-    if (h < kv_heads) inv *= 1.0f / sqrtf((float)dim);
-    for (int d = lane; d < dim; d += WAVE) out[h * dim + d] = src[d] * inv;
+  const int C = unit_heads * dim + heads * vdim;
+  const float* old = state + (long long)slots[e] * state_stride + conv_offset;
+  float* out = qkv + (long long)t * C;
+  const bool unit = seg < unit_heads;
+  const int first = unit ? seg * dim : unit_heads * dim + (seg - unit_heads) * PREP_SPAN;
+  const int last = unit ? first + dim : min(C, first + PREP_SPAN);
+  float kept[PREP_SPAN / 256];      // a segment is at most 1,024 channels: four to a thread
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PREP_SPAN / 256; ++i) {
+    const int c = first + threadIdx.x + i * 256;
+    float y = 0.f;
+    if (c < last) {
+      float sum = 0.f;
+      for (int j = 0; j < taps; ++j)
+        sum = fmaf(conv[(long long)c * taps + j], conv_input(proj, ldp, old, C, taps, t, offset, fresh, taps - 1 - j, c), sum);
+      y = silu_f(sum);
+    }
+    kept[i] = y;
+    ss += y * y;
   }
-  for (int c = unit_heads * dim + threadIdx.x; c < C; c += blockDim.x) out[c] = row[c];
-  for (int h = threadIdx.x; h < heads; h += blockDim.x) {
-    const float* p = proj + (long long)t * ldp;
-    beta[(long long)t * heads + h] = sigmoid_f(p[b_col + h]);
-    decay[(long long)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(p[a_col + h] + dt_bias[h]));
+  float scale = 1.f;
+  if (unit) {       // the same for all threads of the workgroup
+    ss = block_sum(ss, scratch);
+    scale = 1.0f / sqrtf(ss + unit_eps);
+    if (seg < kv_heads) scale *= 1.0f / sqrtf((float)dim);
   }
+#pragma unroll
+  for (int i = 0; i < PREP_SPAN / 256; ++i) {
+    const int c = first + threadIdx.x + i * 256;
+    if (c < last) out[c] = kept[i] * scale;
+  }
+  if (seg == 0)
+    for (int h = threadIdx.x; h < heads; h += blockDim.x) {
+      const float* p = proj + (long long)t * ldp;
+      beta[(long long)t * heads + h] = sigmoid_f(p[b_col + h]);
+      decay[(long long)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(p[a_col + h] + dt_bias[h]));
+    }
 }
 
-// The convolution's inputs of an entry's last taps - 1 tokens become the state.  One workgroup per entry; runs
-// after delta_prepare has read the old rows.
+// The convolution's inputs of an entry's last taps - 1 tokens become the state.  Grid (entries, ceil(C / 256)), a
+// thread per channel; runs after delta_prepare has read the old rows.
 __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict__ proj, long long ldp, int taps, int C,
                                                          float* __restrict__ state, long long state_stride,
                                                          long long conv_offset, const int* __restrict__ entry_start,
                                                          const int* __restrict__ entry_first,
                                                          const int* __restrict__ slots) {
   const int e = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
   const int start = entry_start[e], count = entry_start[e + 1] - start;
   const bool fresh = entry_first[e] == 0;
   float* rows = state + (long long)slots[e] * state_stride + conv_offset;
   const int keep = taps - 1;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    for (int j = 0; j < keep; ++j) {           // ascending: row j + count is read before it is written
-      const int from = j + count;              // index into [old rows (keep) | the entry's tokens (count)]
-      float x;
-      if (from >= keep) x = proj[(long long)(start + from - keep) * ldp + c];
-      else x = fresh ? 0.f : rows[(long long)from * C + c];
-      rows[(long long)j * C + c] = x;
-    }
+  for (int j = 0; j < keep; ++j) {           // ascending: row j + count is read before it is written
+    const int from = j + count;              // index into [old rows (keep) | the entry's tokens (count)]
+    const bool in_step = from >= keep;
+    const float* source = in_step ? proj + (long long)(start + from - keep) * ldp + c : rows + (long long)from * C + c;
+    const float x = *source;
+    rows[(long long)j * C + c] = (in_step || !fresh) ? x : 0.f;
   }
 }
 
@@ -325,7 +339,9 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ 
   const float* saved = state + (long long)slots[e] * state_stride + prev_offset;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float cur = to_float<T>(h[(long long)t * width + c]);
-    const float prev = first ? (fresh ? 0.f : saved[c]) : to_float<T>(h[(long long)(t - 1) * width + c]);
+    // one load from a selected address, masked: no load behind a branch
+    const float before = first ? saved[c] : to_float<T>(h[(long long)(t - 1) * width + c]);
+    const float prev = (first && fresh) ? 0.f : before;
     const float diff = prev - cur;
     for (int s = 0; s < mixes; ++s)
       out[((long long)s * num_tokens + t) * width + c] = from_float<T>(fmaf(diff, mu[(long long)s * width + c], cur));
@@ -378,7 +394,6 @@ __global__ void tanh_kernel(const float* __restrict__ x, TO* __restrict__ out, l
 }
 
 // ---------------------------------------------------------------------------------------------
-static inline bool fits_lds(long long bytes) { return bytes <= 64 * 1024; }
 
 extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* conv, int taps, float* state,
                                 long long state_stride, long long conv_offset, const int* entry_of,
@@ -389,16 +404,17 @@ extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* c
   if (num_tokens <= 0) return 0;
   if (taps < 1 || kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
   const long long C = 2LL * kv_heads * dim + (long long)heads * vdim;
-  if (!fits_lds(C * 4)) return VK_UNSUPPORTED_SIZE;
+  if (dim > PREP_SPAN || C > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-  delta_prepare_kernel<<<num_tokens, 256, (size_t)C * 4, s>>>(proj, ldp, conv, taps, state, state_stride, conv_offset,
-                                                              entry_of, entry_start, entry_first, slots, a_log, dt_bias,
-                                                              kv_heads, dim, heads, vdim, b_col, a_col, unit_eps, qkv,
-                                                              beta, decay);
+  const long long segments = 2LL * kv_heads + ((long long)heads * vdim + PREP_SPAN - 1) / PREP_SPAN;
+  if (segments > 65535) return VK_UNSUPPORTED_SIZE;
+  delta_prepare_kernel<<<dim3(num_tokens, (unsigned)segments), 256, 0, s>>>(
+      proj, ldp, conv, taps, state, state_stride, conv_offset, entry_of, entry_start, entry_first, slots, a_log, dt_bias,
+      kv_heads, dim, heads, vdim, b_col, a_col, unit_eps, qkv, beta, decay);
   VK_LAUNCH_CHECK();
   if (taps > 1) {
-    conv_state_kernel<<<num_entries, 256, 0, s>>>(proj, ldp, taps, (int)C, state, state_stride, conv_offset,
-                                                  entry_start, entry_first, slots);
+    conv_state_kernel<<<dim3(num_entries, (unsigned)((C + 255) / 256)), 256, 0, s>>>(
+        proj, ldp, taps, (int)C, state, state_stride, conv_offset, entry_start, entry_first, slots);
     VK_LAUNCH_CHECK();
   }
   return 0;
