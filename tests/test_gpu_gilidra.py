@@ -134,7 +134,14 @@ ONE_LAYER = {
     "wkv_wide_head": G.single(G.wkv(1, 72, 4), width=40),
     "experts": G.single(G.wkv(1, 8, 4), G.moe(7, 3, 40, 0.75), width=48),
     "experts_all_chosen": G.single(G.wkv(1, 8, 4), G.moe(3, 3, 24, 2.0), width=48),
+    # wider than one tile of the grouped products, one register set of the recurrences, one block of the attention
+    "experts_wide": G.single(G.wkv(1, 8, 4), G.moe(4, 2, 160, 1.0), width=136),
+    "delta_wide_keys": G.single(G.delta(2, 1, 96, 20, 3), width=72),
+    "delta_widest_keys": G.single(G.delta(1, 1, 136, 72, 2), width=72),
+    "wkv_widest_head": G.single(G.wkv(1, 136, 8), width=72),
+    "latent_wide": G.single(G.latent(5, 40, 24, 72, 136, 168, window=150), width=136),
 }
+LONG = {"experts_wide", "latent_wide"}       # these get a prompt of 330 tokens: several tiles per expert and per head
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -143,10 +150,11 @@ def test_a_mechanism_alone_whole_prompt_then_single_tokens(tmp_path, name, dtype
     cfg = ONE_LAYER[name]
     folder = G.make_folder(tmp_path / name, cfg, 11)
     plain_cfg, w = P.load_folder(folder)
-    requests = {0: G.tokens_of(cfg["vocab"], 45, 1), 1: G.tokens_of(cfg["vocab"], 30, 2)}
+    first = 330 if name in LONG else 45
+    requests = {0: G.tokens_of(cfg["vocab"], first, 1), 1: G.tokens_of(cfg["vocab"], 30, 2)}
     want = {r: P.forward(plain_cfg, w, t) for r, t in requests.items()}
     runner = open_runner(folder, dtype)
-    plan = [[(0, 45)], [(1, 19)]] + [[(1, 1)]] * 11
+    plan = [[(0, first)], [(1, 19)]] + [[(1, 1)]] * 11
     check(replay(runner, requests, plan), want, TOL[dtype], name)
     assert runner.cache.check() == "" and runner.cache.live_requests() == 0
 

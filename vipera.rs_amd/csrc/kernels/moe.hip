@@ -335,7 +335,7 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
   hipStream_t s = (hipStream_t)stream;
   const long long pairs = (long long)num_tokens * top;
   if (pairs > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
-  const bool together = num_tokens <= 64;     // sixteen waves route four tokens each at most
+  const bool together = num_tokens <= 16;     // a wave of the one workgroup for every token
   if (!together) {
     moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights);
     VK_LAUNCH_CHECK();

@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict
 //
 // The state of a head lies in memory as the kernel holds it: [value tile of 16][thread of 256][R], so that a
 // lane's R numbers are contiguous and a workgroup reads and writes one contiguous run.  Nobody else reads it.
-constexpr int REC_BLOCK = 16;    // tokens per LDS block
+constexpr int REC_BLOCK = 16;    // tokens per LDS block; 1 for steps of single tokens (few registers, many waves a SIMD)
 constexpr int REC_COLS = 16;     // value channels per workgroup
 
 template <int CTRL>
@@ -139,13 +139,13 @@ __device__ __forceinline__ float row_sum16(float v) {
 
 // Gated delta rule.  Per head, with S [dim, vdim]:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
 // Grid (entries, heads, ceil(vdim / 16)).  An LDS row of a token: [q: 16R | k: 16R | v: 16 | beta, decay].
-template <int R>
+template <int R, int BLOCK>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
     const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
     float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
     const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
     float* __restrict__ out) {
-  constexpr int DP = 16 * R, ROW = 2 * DP + REC_COLS + 2, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  constexpr int DP = 16 * R, ROW = 2 * DP + REC_COLS + 2, COUNT = BLOCK * ROW, LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane & 15, d0 = grp * R;
@@ -181,14 +181,14 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     }
   };
   fetch(start);
-  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+  for (int t0 = start; t0 < end; t0 += BLOCK) {
     __syncthreads();     // the block before has been read
 #pragma unroll
     for (int i = 0; i < LOADS; ++i)
       if (tid + i * 256 < COUNT) rows[tid + i * 256] = held[i];
     __syncthreads();
-    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
-    const int count = min(REC_BLOCK, end - t0);
+    if (t0 + BLOCK < end) fetch(t0 + BLOCK);
+    const int count = min(BLOCK, end - t0);
     // a token's numbers are read from LDS while the token before it is worked on
     float kk[R], qq[R], b, g, val;
     auto read = [&](int j) {
@@ -234,14 +234,14 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
 // RWKV-style time mixing.  Per head, with S [dim, dim]:  o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T,
 // w = exp(-exp(wraw + w0)) per key channel.  r, k, v, wraw are 32-bit [T, heads * dim] with row strides of their own.
 // Grid (entries, heads, ceil(dim / 16)).  An LDS row of a token: [r: 16R | k: 16R | w: 16R | v: 16].
-template <int R>
+template <int R, int BLOCK>
 __global__ __launch_bounds__(256) void wkv_rule_kernel(
     const float* __restrict__ r, long long ldr, const float* __restrict__ k, long long ldk, const float* __restrict__ v,
     long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
     const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
     int heads, float* __restrict__ out) {
-  constexpr int DP = 16 * R, ROW = 3 * DP + REC_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+  constexpr int DP = 16 * R, ROW = 3 * DP + REC_COLS, COUNT = BLOCK * ROW, LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane & 15, d0 = grp * R;
@@ -275,14 +275,14 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
     }
   };
   fetch(start);
-  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+  for (int t0 = start; t0 < end; t0 += BLOCK) {
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < LOADS; ++i)
       if (tid + i * 256 < COUNT) rows[tid + i * 256] = held[i];
     __syncthreads();
-    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
-    const int count = min(REC_BLOCK, end - t0);
+    if (t0 + BLOCK < end) fetch(t0 + BLOCK);
+    const int count = min(BLOCK, end - t0);
     float rr[R], kk[R], ww[R], val;
     auto read = [&](int j) {
       const float* row = rows + j * ROW;
@@ -428,20 +428,25 @@ extern "C" long long vk_recurrent_head_floats(int dim, int vdim) {
 
 extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
                              long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
-                             int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, void* stream) {
+                             int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, int short_entries,
+                             void* stream) {
   if (num_entries <= 0) return 0;
   if (kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   dim3 grid(num_entries, heads, (vdim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
-#define VK_DELTA(R)                                                                                               \
-  delta_rule_kernel<R><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
-                                            kv_heads, dim, heads, vdim, out)
-  if (dim <= 16) VK_DELTA(1);
-  else if (dim <= 32) VK_DELTA(2);
-  else if (dim <= 64) VK_DELTA(4);
-  else if (dim <= 128) VK_DELTA(8);
-  else VK_DELTA(16);
+#define VK_DELTA(R)                                                                                                    \
+  if (short_entries)                                                                                                   \
+    delta_rule_kernel<R, 1><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
+                                                 kv_heads, dim, heads, vdim, out);                                     \
+  else                                                                                                                 \
+    delta_rule_kernel<R, REC_BLOCK><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start,           \
+                                                         entry_first, slots, kv_heads, dim, heads, vdim, out)
+  if (dim <= 16) { VK_DELTA(1); }
+  else if (dim <= 32) { VK_DELTA(2); }
+  else if (dim <= 64) { VK_DELTA(4); }
+  else if (dim <= 128) { VK_DELTA(8); }
+  else { VK_DELTA(16); }
 #undef VK_DELTA
   VK_LAUNCH_CHECK();
   return 0;
@@ -450,20 +455,24 @@ extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* d
 extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv,
                            const float* wraw, long long ldw, const float* w0, const float* bonus, float* state,
                            long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
-                           int dim, int heads, float* out, int num_entries, void* stream) {
+                           int dim, int heads, float* out, int num_entries, int short_entries, void* stream) {
   if (num_entries <= 0) return 0;
   if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   dim3 grid(num_entries, heads, (dim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
-#define VK_WKV(R)                                                                                                  \
-  wkv_rule_kernel<R><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,       \
-                                          entry_start, entry_first, slots, dim, heads, out)
-  if (dim <= 16) VK_WKV(1);
-  else if (dim <= 32) VK_WKV(2);
-  else if (dim <= 64) VK_WKV(4);
-  else if (dim <= 128) VK_WKV(8);
-  else VK_WKV(16);
+#define VK_WKV(R)                                                                                                     \
+  if (short_entries)                                                                                                  \
+    wkv_rule_kernel<R, 1><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,     \
+                                               entry_start, entry_first, slots, dim, heads, out);                     \
+  else                                                                                                                \
+    wkv_rule_kernel<R, REC_BLOCK><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state,            \
+                                                       state_stride, entry_start, entry_first, slots, dim, heads, out)
+  if (dim <= 16) { VK_WKV(1); }
+  else if (dim <= 32) { VK_WKV(2); }
+  else if (dim <= 64) { VK_WKV(4); }
+  else if (dim <= 128) { VK_WKV(8); }
+  else { VK_WKV(16); }
 #undef VK_WKV
   VK_LAUNCH_CHECK();
   return 0;

@@ -977,8 +977,9 @@ def delta_prepare(proj: torch.Tensor, conv: torch.Tensor, state: torch.Tensor, c
 
 def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
                entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, kv_heads: int, dim: int,
-               heads: int, vdim: int, out: torch.Tensor, num_entries: int) -> None:
-    """The gated delta rule over every entry's tokens in order, from and into the entries' state rows (the first
+               heads: int, vdim: int, out: torch.Tensor, num_entries: int, short_entries: bool = False) -> None:
+    """The gated delta rule over every entry's tokens in order (``short_entries``: a step of single tokens, which
+    takes the kernel's form with few registers; the result is the same), from and into the entries' state rows (the first
     ``heads * recurrent_head_floats(dim, vdim)`` floats of a row, in the kernel's own order); ``out`` 32-bit ``[tokens, heads * vdim]``."""
     _dev(qkv, beta, decay, state, entry_start, entry_first, slots, out)
     tokens = qkv.shape[0]
@@ -992,14 +993,16 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
     _entries_ok((entry_start, entry_first, slots), num_entries)
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"delta_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
-    fn = _fn("recurrent", "vk_delta_rule", [_p, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _i, _p])
+    fn = _fn("recurrent", "vk_delta_rule", [_p, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p])
     _status(fn(_ptr(qkv), _ptr(beta), _ptr(decay), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first),
-               _ptr(slots), kv_heads, dim, heads, vdim, _ptr(out), num_entries, _stream()), "delta_rule")
+               _ptr(slots), kv_heads, dim, heads, vdim, _ptr(out), num_entries, 1 if short_entries else 0, _stream()),
+            "delta_rule")
 
 
 def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor,
              bonus: torch.Tensor, state: torch.Tensor, entry_start: torch.Tensor, entry_first: torch.Tensor,
-             slots: torch.Tensor, dim: int, heads: int, out: torch.Tensor, num_entries: int) -> None:
+             slots: torch.Tensor, dim: int, heads: int, out: torch.Tensor, num_entries: int,
+             short_entries: bool = False) -> None:
     """RWKV-style time mixing over every entry's tokens in order: ``o = (S + diag(u) k v^T)^T r``, then
     ``S = diag(w) S + k v^T`` with ``w = exp(-exp(wraw + w0))``.  ``r, k, v, wraw``: 32-bit ``[tokens, heads * dim]``
     (row-strided views are fine); state rows start with the heads' matrices
@@ -1018,10 +1021,10 @@ def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tens
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"wkv_rule: a head width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
     fn = _fn("recurrent", "vk_wkv_rule",
-             [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _p, _i, _p])
+             [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _p, _i, _i, _p])
     _status(fn(_ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(wraw), wraw.stride(0), _ptr(w0),
                _ptr(bonus), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first), _ptr(slots), dim, heads,
-               _ptr(out), num_entries, _stream()), "wkv_rule")
+               _ptr(out), num_entries, 1 if short_entries else 0, _stream()), "wkv_rule")
 
 
 def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_offset: int, entry_of: torch.Tensor,

@@ -111,7 +111,7 @@ class GatedDelta(Mixer):
                               self.heads, self.vdim, b_col, b_col + self.heads, UNIT_EPS, qkv, beta, decay, entries)
         o = torch.empty((tokens, self.vw), **f32)
         kernels.delta_rule(qkv, beta, decay, state, batch.entry_start, batch.entry_first_pos, batch.slots,
-                           self.kv_heads, self.dim, self.heads, self.vdim, o, entries)
+                           self.kv_heads, self.dim, self.heads, self.vdim, o, entries, short_entries=batch.all_single)
         gated = self.runtime.empty((tokens, self.vw))
         kernels.head_norm_gate(o, self.norm, proj[:, g_col:g_col + self.vw], True, self.eps, self.heads, self.vdim, gated)
         linear(gated, self.w_o, None, residual, accumulate=True)
@@ -190,7 +190,7 @@ class Wkv(Mixer):
         linear(squashed, self.w2, None, wraw)
         o = torch.empty((tokens, self.width), **f32)
         kernels.wkv_rule(rkv[0], rkv[1], rkv[2], wraw, self.w0, self.bonus, state, batch.entry_start,
-                         batch.entry_first_pos, batch.slots, self.dim, self.heads, o, entries)
+                         batch.entry_first_pos, batch.slots, self.dim, self.heads, o, entries, short_entries=batch.all_single)
         gated = self.runtime.empty((tokens, self.width))
         kernels.head_norm_gate(o, self.norm, gate, True, self.eps, self.heads, self.dim, gated)
         linear(gated, self.w_o, None, residual, accumulate=True)
