@@ -140,6 +140,7 @@ ONE_LAYER = {
     "delta_widest_keys": G.single(G.delta(1, 1, 136, 72, 2), width=72),
     "wkv_widest_head": G.single(G.wkv(1, 136, 8), width=72),
     "latent_wide": G.single(G.latent(5, 40, 24, 72, 136, 168, window=150), width=136),
+    "latent_many_heads": G.single(G.latent(20, 8, 8, 8, 16, 24, window=23), width=40),    # more than one block of query heads
 }
 LONG = {"experts_wide", "latent_wide"}       # these get a prompt of 330 tokens: several tiles per expert and per head
 
@@ -329,6 +330,26 @@ def test_greedy_generation_through_the_engine(g1, dtype, graphs, pipelined):
     if graphs:
         assert engine.runner.graphs.replays > 0
     assert engine.runner.cache.check() == "" and engine.runner.cache.live_requests() == 0
+
+
+def test_the_command_line_generates(g2):
+    """``bin/vipera generate`` on a Gilidra folder: the model is found by its configuration and run through the engine."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    folder, cfg, w = g2
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prompt = G.tokens_of(cfg["vocab"], 11, 3)
+    done = subprocess.run([sys.executable, os.path.join(root, "bin", "vipera"), "generate", folder, "--prompt-ids",
+                           " ".join(str(t) for t in prompt), "--max-tokens", "8", "--dtype", "float32", "--json"],
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-2000:]
+    report = json.loads(done.stdout)
+    assert report["prompt_tokens"] == 11 and report["generated_tokens"] == 8
+    logits = P.forward(cfg, w, prompt + report["tokens"][:-1])
+    assert assert_tokens_follow_plain(logits, len(prompt), report["tokens"], 2.5e-5, "command line") >= 4
 
 
 def test_the_trace_runner_replays_a_schedule(tmp_path, g2):

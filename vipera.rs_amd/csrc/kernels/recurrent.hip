@@ -337,7 +337,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const T* __restrict__ 
   const bool first = t == entry_start[e];
   const bool fresh = entry_first[e] == 0;
   const float* saved = state + (long long)slots[e] * state_stride + prev_offset;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     const float cur = to_float<T>(h[(long long)t * width + c]);
     // one load from a selected address, masked: no load behind a branch
     const float before = first ? saved[c] : to_float<T>(h[(long long)(t - 1) * width + c]);
@@ -357,7 +357,8 @@ __global__ __launch_bounds__(256) void save_last_kernel(const T* __restrict__ h,
   const int e = blockIdx.x;
   const int last = entry_start[e + 1] - 1;
   float* saved = state + (long long)slots[e] * state_stride + prev_offset;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) saved[c] = to_float<T>(h[(long long)last * width + c]);
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x)
+    saved[c] = to_float<T>(h[(long long)last * width + c]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -485,19 +486,22 @@ extern "C" int vk_token_shift(const void* h, int dtype, int width, const float* 
   if (num_tokens <= 0) return 0;
   if (width < 1 || mixes < 1) return VK_BAD_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
+  // a step of few tokens spreads a row over several workgroups; a prompt's many tokens fill the GPU by themselves
+  const unsigned spans = num_tokens >= 512 ? 1u : (unsigned)min(64, (width + 255) / 256);
+  const dim3 tokens_grid(num_tokens, spans), entries_grid(num_entries, spans);
   if (dtype == DT_F32) {
-    token_shift_kernel<float><<<num_tokens, 256, 0, s>>>((const float*)h, width, mu, mixes, state, state_stride,
+    token_shift_kernel<float><<<tokens_grid, 256, 0, s>>>((const float*)h, width, mu, mixes, state, state_stride,
                                                          prev_offset, entry_of, entry_start, entry_first, slots,
                                                          num_tokens, (float*)out);
     VK_LAUNCH_CHECK();
-    save_last_kernel<float><<<num_entries, 256, 0, s>>>((const float*)h, width, state, state_stride, prev_offset,
+    save_last_kernel<float><<<entries_grid, 256, 0, s>>>((const float*)h, width, state, state_stride, prev_offset,
                                                         entry_start, slots);
   } else if (dtype == DT_BF16) {
-    token_shift_kernel<bf16_t><<<num_tokens, 256, 0, s>>>((const bf16_t*)h, width, mu, mixes, state, state_stride,
+    token_shift_kernel<bf16_t><<<tokens_grid, 256, 0, s>>>((const bf16_t*)h, width, mu, mixes, state, state_stride,
                                                           prev_offset, entry_of, entry_start, entry_first, slots,
                                                           num_tokens, (bf16_t*)out);
     VK_LAUNCH_CHECK();
-    save_last_kernel<bf16_t><<<num_entries, 256, 0, s>>>((const bf16_t*)h, width, state, state_stride, prev_offset,
+    save_last_kernel<bf16_t><<<entries_grid, 256, 0, s>>>((const bf16_t*)h, width, state, state_stride, prev_offset,
                                                          entry_start, slots);
   } else {
     return VK_BAD_ARGUMENT;
