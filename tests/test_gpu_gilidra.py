@@ -193,6 +193,22 @@ def g2(tmp_path_factory):
     return (folder,) + P.load_folder(folder)
 
 
+# every width odd in some way: nothing is a multiple of 8, the model's width not even of 4
+G3 = G.config(83, 50, [G.wkv(3, 10, 6), G.latent(3, 6, 6, 10, 14, 22, window=9), G.delta(3, 1, 10, 14, 3)],
+              [G.moe(5, 2, 18, 1.0), G.moe(3, 1, 22, 1.0), G.moe(5, 2, 18, 1.0)], logit_scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_widths_that_fit_no_fast_path(tmp_path, dtype):
+    folder = G.make_folder(tmp_path / "g3", G3, 41)
+    cfg, w = P.load_folder(folder)
+    requests = {0: G.tokens_of(cfg["vocab"], 40, 1), 1: G.tokens_of(cfg["vocab"], 21, 2)}
+    want = {r: P.forward(cfg, w, t) for r, t in requests.items()}
+    runner = open_runner(folder, dtype, page=4)
+    plan = [[(0, 17), (1, 2)], [(0, 2), (1, 1)], [(0, 21), (1, 1)]] + [[(1, 1)]] * 17
+    check(replay(runner, requests, plan), want, TOL[dtype], "odd widths")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("which", ["g1", "g2"])
 def test_token_by_token_equals_the_whole_prompt(request, which, dtype):

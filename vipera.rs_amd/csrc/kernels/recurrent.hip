@@ -117,8 +117,12 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict
 // blocks of 16: a block's k, q (or r, k, decay), values and gates are fetched into registers while the block before
 // is worked on, and passed on through LDS, so that a token's step waits for no memory.
 //
-// The state of a head lies in memory as the kernel holds it: [value tile of 16][thread of 256][R], so that a
-// lane's R numbers are contiguous and a workgroup reads and writes one contiguous run.  Nobody else reads it.
+// This form runs the steps of single tokens (BLOCK 1: few registers, many waves a SIMD); prompts' portions run on
+// the scan kernels further down, a wave to a value channel.
+//
+// The state of a head lies in memory as [value channel, padded to 16][key channel, padded to 16 R]: a lane's R
+// numbers are contiguous, a row's sixteen lanes hold one value channel's run, and a workgroup reads and writes one
+// contiguous run.  Both forms read it; nobody else does.
 constexpr int REC_BLOCK = 16;    // tokens per LDS block; 1 for steps of single tokens (few registers, many waves a SIMD)
 constexpr int REC_COLS = 16;     // value channels per workgroup
 
@@ -154,7 +158,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
   const int kh = h / (heads / kv_heads);
   const int C = 2 * kv_heads * dim + heads * vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
-  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z + blockIdx.z) * 256 + tid) * R;
+  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z * REC_COLS + v) * 16 + grp) * R;
   const bool fresh = entry_first[e] == 0;
   float S[R];
 #pragma unroll
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
   const int v0 = blockIdx.z * REC_COLS, mine_col = wave * 4 + (lane >> 4), col_v = v0 + mine_col;
   const bool live = col_v < dim;
   const int start = entry_start[e], end = entry_start[e + 1];
-  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z + blockIdx.z) * 256 + tid) * R;
+  float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z * REC_COLS + col_v) * 16 + grp) * R;
   const bool fresh = entry_first[e] == 0;
   float S[R], U[R];
 #pragma unroll
@@ -318,6 +322,188 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
   }
 #pragma unroll
   for (int i = 0; i < R; ++i) mine[i] = S[i];
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same recurrences for prompts' portions: a wave owns ONE value channel and its 64 lanes the key channels, Q of
+// them each (64 Q >= the state's padded key width), so that one prompt of a few thousand tokens is heads x value
+// channels waves, two or more to a SIMD, each with a short step per token: Q terms a lane, four DPP exchanges inside
+// the rows, and the four rows' sums read by every lane.  A workgroup is eight waves (eight value channels) that share a
+// block's k, q (r, k, decay) in LDS.  What a thread fetches of a block is worked out once, before the first block.
+constexpr int SCAN_COLS = 8;
+constexpr int SCAN_THREADS = SCAN_COLS * 64;
+
+__device__ __forceinline__ float wave_total(float v) {
+  v = row_sum16(v);
+  const int bits = __float_as_int(v);
+  return __int_as_float(__builtin_amdgcn_readlane(bits, 0)) + __int_as_float(__builtin_amdgcn_readlane(bits, 16)) +
+         (__int_as_float(__builtin_amdgcn_readlane(bits, 32)) + __int_as_float(__builtin_amdgcn_readlane(bits, 48)));
+}
+
+// A block's fetch plan: element x = tid + i * SCAN_THREADS of the block is token x / ROW, column x % ROW; `plan[i]` is
+// token * 2^24 + the column's offset inside the token's row of the source, or -1 for an element that is always zero.
+template <int Q>
+__global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
+    float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
+    const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
+    int key_pad, int value_pad, float* __restrict__ out) {
+  constexpr int DP = 64 * Q, ROW = 2 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
+  __shared__ float rows[COUNT];
+  __shared__ float gates[REC_BLOCK][2];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int d0 = lane * Q;
+  const int v0 = blockIdx.z * SCAN_COLS, v = v0 + wave;
+  const bool live = v < vdim;
+  const int kh = h / (heads / kv_heads);
+  const int C = 2 * kv_heads * dim + heads * vdim;
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * value_pad + v) * key_pad + d0;
+  const bool fresh = entry_first[e] == 0, kept = v < value_pad;
+  float S[Q];
+#pragma unroll
+  for (int i = 0; i < Q; ++i) S[i] = (!fresh && kept && d0 + i < key_pad) ? mine[i] : 0.f;
+  int plan[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int x = tid + i * SCAN_THREADS, j = x / ROW, col = x % ROW;
+    int within = -1;
+    if (x < COUNT) {
+      if (col < DP) { if (col < dim) within = kh * dim + col; }
+      else if (col < 2 * DP) { if (col - DP < dim) within = (kv_heads + kh) * dim + col - DP; }
+      else if (v0 + col - 2 * DP < vdim) within = 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP;
+    }
+    plan[i] = within < 0 ? -1 : (j << 24) | within;
+  }
+  float held[LOADS], held_gate = 0.f;
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      // a token past the entry's end is never worked on: its address is clamped, its value does not matter
+      const int t = min(t0 + (plan[i] >> 24 & 127), end - 1);
+      const float loaded = qkv[(long long)t * C + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
+      held[i] = plan[i] < 0 ? 0.f : loaded;
+    }
+    if (tid < 2 * REC_BLOCK) {
+      const int t = min(t0 + (tid >> 1), end - 1);
+      held_gate = ((tid & 1) ? decay : beta)[(long long)t * heads + h];
+    }
+  };
+  fetch(start);
+  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+    __syncthreads();     // the block before has been read
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+    if (tid < 2 * REC_BLOCK) gates[tid >> 1][tid & 1] = held_gate;
+    __syncthreads();
+    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    const int count = min(REC_BLOCK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float* row = rows + j * ROW;
+      const float b = gates[j][0], g = gates[j][1], val = row[2 * DP + wave];
+      float kk[Q], qq[Q];
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        kk[i] = row[DP + d0 + i];
+        qq[i] = row[d0 + i];
+      }
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        S[i] *= g;
+        dot = fmaf(S[i], kk[i], dot);
+      }
+      const float u = b * (val - wave_total(dot));
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        S[i] = fmaf(kk[i], u, S[i]);
+        o = fmaf(S[i], qq[i], o);
+      }
+      o = wave_total(o);
+      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = o;
+    }
+  }
+  if (kept) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i)
+      if (d0 + i < key_pad) mine[i] = S[i];
+  }
+}
+
+// An LDS row of a token: [r: 64Q | k: 64Q | w: 64Q | v: 8]; sources differ by column, so the plan keeps which.
+template <int Q>
+__global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
+    const float* __restrict__ r, long long ldr, const float* __restrict__ k, long long ldk, const float* __restrict__ v,
+    long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
+    const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
+    int heads, int key_pad, int value_pad, float* __restrict__ out) {
+  constexpr int DP = 64 * Q, ROW = 3 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
+  __shared__ float rows[COUNT];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int d0 = lane * Q;
+  const int v0 = blockIdx.z * SCAN_COLS, col_v = v0 + wave;
+  const bool live = col_v < dim;
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* mine = state + (long long)slots[e] * state_stride + ((long long)h * value_pad + col_v) * key_pad + d0;
+  const bool fresh = entry_first[e] == 0, kept = col_v < value_pad;
+  float S[Q], U[Q];
+#pragma unroll
+  for (int i = 0; i < Q; ++i) {
+    S[i] = (!fresh && kept && d0 + i < key_pad) ? mine[i] : 0.f;
+    U[i] = d0 + i < dim ? bonus[h * dim + d0 + i] : 0.f;
+  }
+  // kind * 2^28 + token * 2^21 + offset inside the head's dim (kinds: 0 r, 1 k, 2 decay, 3 value), or -1
+  int plan[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int x = tid + i * SCAN_THREADS, j = x / ROW, col = x % ROW;
+    const int kind = col < DP ? 0 : col < 2 * DP ? 1 : col < 3 * DP ? 2 : 3;
+    const int d = kind < 3 ? col - kind * DP : v0 + col - 3 * DP;
+    plan[i] = (x < COUNT && d < dim) ? (kind << 28) | (j << 21) | d : -1;
+  }
+  float held[LOADS];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int kind = plan[i] >> 28 & 3, d = plan[i] < 0 ? 0 : plan[i] & 0x1FFFFF;
+      const long long t = min(t0 + (plan[i] >> 21 & 127), end - 1);
+      const float* base = kind == 0 ? r + t * ldr : kind == 1 ? k + t * ldk : kind == 2 ? wraw + t * ldw : v + t * ldv;
+      const float loaded = base[h * dim + d];
+      const float shift = w0[h * dim + d];
+      held[i] = plan[i] < 0 ? 0.f : kind == 2 ? expf(-expf(loaded + shift)) : loaded;
+    }
+  };
+  fetch(start);
+  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+    __syncthreads();
+    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    const int count = min(REC_BLOCK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float* row = rows + j * ROW;
+      const float val = row[3 * DP + wave];
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        const float kv = row[DP + d0 + i] * val;
+        o = fmaf(fmaf(U[i], kv, S[i]), row[d0 + i], o);
+        S[i] = fmaf(row[2 * DP + d0 + i], S[i], kv);
+      }
+      o = wave_total(o);
+      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = o;
+    }
+  }
+  if (kept) {
+#pragma unroll
+    for (int i = 0; i < Q; ++i)
+      if (d0 + i < key_pad) mine[i] = S[i];
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -421,10 +607,12 @@ extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* c
   return 0;
 }
 
-// Floats of one head's state as the recurrence kernels lay it out: value tiles of 16 x 256 threads x R.
+// Key channels a lane of the single-token form keeps: the state's key width is padded to 16 times this.
+static inline int rows_of(int dim) { return dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
+
+// Floats of one head's state as the recurrence kernels lay it out: [value channels padded to 16][key channels padded].
 extern "C" long long vk_recurrent_head_floats(int dim, int vdim) {
-  const int r = dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16;
-  return (long long)((vdim + REC_COLS - 1) / REC_COLS) * 256 * r;
+  return (long long)((vdim + REC_COLS - 1) / REC_COLS) * REC_COLS * 16 * rows_of(dim);
 }
 
 extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
@@ -436,13 +624,23 @@ extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* d
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   dim3 grid(num_entries, heads, (vdim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
+  const int key_pad = 16 * rows_of(dim), value_pad = (vdim + REC_COLS - 1) / REC_COLS * REC_COLS;
+  if (!short_entries) {
+    dim3 scan_grid(num_entries, heads, value_pad / SCAN_COLS);
+#define VK_DELTA_SCAN(Q)                                                                                             \
+  delta_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start,         \
+                                                          entry_first, slots, kv_heads, dim, heads, vdim, key_pad,    \
+                                                          value_pad, out)
+    if (key_pad <= 64) VK_DELTA_SCAN(1);
+    else if (key_pad <= 128) VK_DELTA_SCAN(2);
+    else VK_DELTA_SCAN(4);
+#undef VK_DELTA_SCAN
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
 #define VK_DELTA(R)                                                                                                    \
-  if (short_entries)                                                                                                   \
-    delta_rule_kernel<R, 1><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
-                                                 kv_heads, dim, heads, vdim, out);                                     \
-  else                                                                                                                 \
-    delta_rule_kernel<R, REC_BLOCK><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start,           \
-                                                         entry_first, slots, kv_heads, dim, heads, vdim, out)
+  delta_rule_kernel<R, 1><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
+                                               kv_heads, dim, heads, vdim, out)
   if (dim <= 16) { VK_DELTA(1); }
   else if (dim <= 32) { VK_DELTA(2); }
   else if (dim <= 64) { VK_DELTA(4); }
@@ -462,13 +660,23 @@ extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long l
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   dim3 grid(num_entries, heads, (dim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
+  const int key_pad = 16 * rows_of(dim), value_pad = (dim + REC_COLS - 1) / REC_COLS * REC_COLS;
+  if (!short_entries) {
+    dim3 scan_grid(num_entries, heads, value_pad / SCAN_COLS);
+#define VK_WKV_SCAN(Q)                                                                                               \
+  wkv_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state,          \
+                                                        state_stride, entry_start, entry_first, slots, dim, heads,    \
+                                                        key_pad, value_pad, out)
+    if (key_pad <= 64) VK_WKV_SCAN(1);
+    else if (key_pad <= 128) VK_WKV_SCAN(2);
+    else VK_WKV_SCAN(4);
+#undef VK_WKV_SCAN
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
 #define VK_WKV(R)                                                                                                     \
-  if (short_entries)                                                                                                  \
-    wkv_rule_kernel<R, 1><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,     \
-                                               entry_start, entry_first, slots, dim, heads, out);                     \
-  else                                                                                                                \
-    wkv_rule_kernel<R, REC_BLOCK><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state,            \
-                                                       state_stride, entry_start, entry_first, slots, dim, heads, out)
+  wkv_rule_kernel<R, 1><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,       \
+                                             entry_start, entry_first, slots, dim, heads, out)
   if (dim <= 16) { VK_WKV(1); }
   else if (dim <= 32) { VK_WKV(2); }
   else if (dim <= 64) { VK_WKV(4); }
