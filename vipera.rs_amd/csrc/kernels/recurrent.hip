@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
     long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
     const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
-    int heads, float* __restrict__ out) {
+    int heads, int decayed, float* __restrict__ out) {
   constexpr int DP = 16 * R, ROW = 3 * DP + REC_COLS, COUNT = BLOCK * ROW, LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(256) void wkv_rule_kernel(
       const int within = ok ? h * dim + ((is_r || is_k || is_w) ? d : v0 + c) : 0;
       const float loaded = base[within];
       const float shift = w0[(ok && is_w) ? h * dim + d : 0];
-      const float value = !ok ? 0.f : is_w ? expf(-expf(loaded + shift)) : loaded;
+      const float value = !ok ? 0.f : (is_w && !decayed) ? expf(-expf(loaded + shift)) : loaded;
       held[i] = value;
     }
   };
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
     long long ldv, const float* __restrict__ wraw, long long ldw, const float* __restrict__ w0,
     const float* __restrict__ bonus, float* __restrict__ state, long long state_stride,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
-    int heads, int key_pad, int value_pad, float* __restrict__ out) {
+    int heads, int key_pad, int value_pad, int decayed, float* __restrict__ out) {
   constexpr int DP = 64 * Q, ROW = 3 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -471,9 +471,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
       const int kind = plan[i] >> 28 & 3, d = plan[i] < 0 ? 0 : plan[i] & 0x1FFFFF;
       const long long t = min(t0 + (plan[i] >> 21 & 127), end - 1);
       const float* base = kind == 0 ? r + t * ldr : kind == 1 ? k + t * ldk : kind == 2 ? wraw + t * ldw : v + t * ldv;
-      const float loaded = base[h * dim + d];
-      const float shift = w0[h * dim + d];
-      held[i] = plan[i] < 0 ? 0.f : kind == 2 ? expf(-expf(loaded + shift)) : loaded;
+      float loaded = base[h * dim + d];
+      if (!decayed) {      // the same for every thread: the caller has not turned wraw into the decay yet
+        const float shift = w0[h * dim + d];
+        loaded = kind == 2 ? expf(-expf(loaded + shift)) : loaded;
+      }
+      held[i] = plan[i] < 0 ? 0.f : loaded;
     }
   };
   fetch(start);
@@ -573,6 +576,12 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   }
 }
 
+// x[t, c] = exp(-exp(x[t, c] + w0[c])) in place: time mixing's decay, for a step whose recurrence reads it many times.
+__global__ void decay_kernel(float* __restrict__ x, const float* __restrict__ w0, int width, long long count) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) x[i] = expf(-expf(x[i] + w0[i % width]));
+}
+
 // out = tanh(x), elementwise, 32-bit in, TO out.
 template <typename TO>
 __global__ void tanh_kernel(const float* __restrict__ x, TO* __restrict__ out, long long count) {
@@ -654,7 +663,8 @@ extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* d
 extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv,
                            const float* wraw, long long ldw, const float* w0, const float* bonus, float* state,
                            long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
-                           int dim, int heads, float* out, int num_entries, int short_entries, void* stream) {
+                           int dim, int heads, float* out, int num_entries, int short_entries, int decayed,
+                           void* stream) {
   if (num_entries <= 0) return 0;
   if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
@@ -666,7 +676,7 @@ extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long l
 #define VK_WKV_SCAN(Q)                                                                                               \
   wkv_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state,          \
                                                         state_stride, entry_start, entry_first, slots, dim, heads,    \
-                                                        key_pad, value_pad, out)
+                                                        key_pad, value_pad, decayed, out)
     if (key_pad <= 64) VK_WKV_SCAN(1);
     else if (key_pad <= 128) VK_WKV_SCAN(2);
     else VK_WKV_SCAN(4);
@@ -676,7 +686,7 @@ extern "C" int vk_wkv_rule(const float* r, long long ldr, const float* k, long l
   }
 #define VK_WKV(R)                                                                                                     \
   wkv_rule_kernel<R, 1><<<grid, 256, 0, s>>>(r, ldr, k, ldk, v, ldv, wraw, ldw, w0, bonus, state, state_stride,       \
-                                             entry_start, entry_first, slots, dim, heads, out)
+                                             entry_start, entry_first, slots, dim, heads, decayed, out)
   if (dim <= 16) { VK_WKV(1); }
   else if (dim <= 32) { VK_WKV(2); }
   else if (dim <= 64) { VK_WKV(4); }
@@ -735,6 +745,14 @@ extern "C" int vk_head_norm_gate(const float* o, const float* weight, int weight
   else if (gate_dtype == DT_BF16 && out_dtype == DT_F32) VK_HNG(bf16_t, float);
   else return VK_BAD_ARGUMENT;
 #undef VK_HNG
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_decay(float* x, const float* w0, int width, long long count, void* stream) {
+  if (count <= 0) return 0;
+  if (width < 1) return VK_BAD_ARGUMENT;
+  decay_kernel<<<(unsigned)((count + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, w0, width, count);
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -915,6 +915,15 @@ def scale_(x: torch.Tensor, factor: float) -> None:
     _status(fn(_ptr(x), float(factor), x.numel(), _stream()), "scale")
 
 
+def decay_(x: torch.Tensor, w0: torch.Tensor) -> None:
+    """``x = exp(-exp(x + w0))`` in place; ``x`` 32-bit ``[tokens, width]``, ``w0`` ``[width]``."""
+    _dev(x, w0)
+    _f32(x, "decay: x")
+    _need(x.dim() == 2 and w0.dtype == torch.float32 and w0.is_contiguous() and w0.numel() == x.shape[1], "decay: w0")
+    fn = _fn("recurrent", "vk_decay", [_p, _p, _i, _ll, _p])
+    _status(fn(_ptr(x), _ptr(w0), x.shape[1], x.numel(), _stream()), "decay")
+
+
 def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
     """``out = tanh(x)``; ``x`` 32-bit, ``out`` of either dtype."""
     _dev(x, out)
@@ -1002,11 +1011,12 @@ def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state
 def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor,
              bonus: torch.Tensor, state: torch.Tensor, entry_start: torch.Tensor, entry_first: torch.Tensor,
              slots: torch.Tensor, dim: int, heads: int, out: torch.Tensor, num_entries: int,
-             short_entries: bool = False) -> None:
+             short_entries: bool = False, decayed: bool = False) -> None:
     """RWKV-style time mixing over every entry's tokens in order: ``o = (S + diag(u) k v^T)^T r``, then
     ``S = diag(w) S + k v^T`` with ``w = exp(-exp(wraw + w0))``.  ``r, k, v, wraw``: 32-bit ``[tokens, heads * dim]``
     (row-strided views are fine); state rows start with the heads' matrices
-    (``heads * recurrent_head_floats(dim, dim)`` floats, in the kernel's own order)."""
+    (``heads * recurrent_head_floats(dim, dim)`` floats, in the kernel's own order).  ``decayed``: ``wraw`` already
+    holds ``w`` (see :func:`decay_`)."""
     _dev(r, k, v, wraw, w0, bonus, state, entry_start, entry_first, slots, out)
     tokens, width = out.shape[0], heads * dim
     for name, t in (("r", r), ("k", k), ("v", v), ("wraw", wraw)):
@@ -1021,10 +1031,10 @@ def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tens
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"wkv_rule: a head width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
     fn = _fn("recurrent", "vk_wkv_rule",
-             [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _p, _i, _i, _p])
+             [_p, _ll, _p, _ll, _p, _ll, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _p, _i, _i, _i, _p])
     _status(fn(_ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(wraw), wraw.stride(0), _ptr(w0),
                _ptr(bonus), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first), _ptr(slots), dim, heads,
-               _ptr(out), num_entries, 1 if short_entries else 0, _stream()), "wkv_rule")
+               _ptr(out), num_entries, 1 if short_entries else 0, 1 if decayed else 0, _stream()), "wkv_rule")
 
 
 def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_offset: int, entry_of: torch.Tensor,

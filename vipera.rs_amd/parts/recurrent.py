@@ -189,8 +189,14 @@ class Wkv(Mixer):
         wraw = torch.empty((tokens, self.width), **f32)
         linear(squashed, self.w2, None, wraw)
         o = torch.empty((tokens, self.width), **f32)
+        # a prompt's recurrence reads a token's decay once per workgroup of value channels: the two exponentials are
+        # taken once, ahead of it; a step of single tokens takes them inside the recurrence (one launch less)
+        ahead = not batch.all_single
+        if ahead:
+            kernels.decay_(wraw, self.w0)
         kernels.wkv_rule(rkv[0], rkv[1], rkv[2], wraw, self.w0, self.bonus, state, batch.entry_start,
-                         batch.entry_first_pos, batch.slots, self.dim, self.heads, o, entries, short_entries=batch.all_single)
+                         batch.entry_first_pos, batch.slots, self.dim, self.heads, o, entries,
+                         short_entries=batch.all_single, decayed=ahead)
         gated = self.runtime.empty((tokens, self.width))
         kernels.head_norm_gate(o, self.norm, gate, True, self.eps, self.heads, self.dim, gated)
         linear(gated, self.w_o, None, residual, accumulate=True)
