@@ -158,7 +158,7 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 // unrolling): a wave has few steps and memory is the bound.
 template <bool REGS>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
-                                             const CacheView& cv, float scale, f32x4 (&o)[DT], float& m, float& l) {
+                                             const CacheView& cv, float scale, float softcap, f32x4 (&o)[DT], float& m, float& l) {
   const int lane = threadIdx.x & 63, lg = lane >> 4;
   const int first = begin & ~31;
   if (first >= end) return;
@@ -186,7 +186,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       for (int j = 0; j < 4; ++j) {
         const int p = kb + lg * 8 + sub * 4 + j;
         const bool visible = p >= col_lo && p <= col_pos && p >= begin && p < end;
-        const float x = visible ? s[sub][j] * scale : -INFINITY;
+        const float x = visible ? capped(s[sub][j] * scale, softcap) : -INFINITY;
         sv[sub * 4 + j] = x;
         tile_max = fmaxf(tile_max, x);
       }
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, int cus) {
+    float scale, int window, float softcap, int cus) {
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];
   __bf16* sK = lds;                     // [PT_KV][PT_KROW]
   __bf16* sV = lds + PT_KV * PT_KROW;   // [HDP][PT_VROW]
@@ -275,7 +275,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // the workgroup's range of positions
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = first_pos + tile_off;
-  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int begin = first_visible(tile_first_pos, window);
   const int end = tile_first_pos + tile_cols;  // one past the last column's position
 
   // this wave's columns
@@ -283,15 +283,15 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   const int c = q_off + lr;
   const bool col_ok = c < count;
   const int col_pos = col_ok ? first_pos + c : -1;
-  const int col_lo = (window > 0 && col_pos + 1 > window) ? col_pos + 1 - window : 0;
+  const int col_lo = first_visible(col_pos, window);
   bf16x8 qf[KS];
   load_q(col_ok ? q + (size_t)(tok0 + c) * q_stride + (size_t)h * hd : nullptr, hd, qf);
   const int wave_cols = max(0, min(16, count - q_off));
   const int wave_end = wave_cols > 0 ? first_pos + q_off + wave_cols : 0;  // nothing at or past it is visible
   const int wave_first = first_pos + q_off;
-  const int wave_begin = (window > 0 && wave_first + 1 > window) ? wave_first + 1 - window : 0;
+  const int wave_begin = first_visible(wave_first, window);
   const int wave_last = wave_end - 1;  // position of the wave's last column
-  const int wave_lo_max = (window > 0 && wave_last + 1 > window) ? wave_last + 1 - window : 0;
+  const int wave_lo_max = first_visible(wave_last, window);
 
   f32x4 o[DT];
   float m = -INFINITY, l = 0.f;
@@ -397,6 +397,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // comparisons. The sums are rescaled only when some column's maximum moved, which is rare after the
   // first tiles.
   const float c2 = scale * 1.44269504088896341f;
+  const float cap_raw = softcap > 0.f ? softcap / scale : 0.f, cap_inv = softcap > 0.f ? scale / softcap : 0.f;
   auto tile_body = [&](bool masked, int p0) {
     // ---- scores of four 16-position tiles
     f32x4 s[4];
@@ -409,6 +410,12 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
       }
       s[sub] = acc;
+    }
+    if (softcap > 0.f) {   // raw scores whose product with the scale is the capped score
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[sub][j] = cap_raw * tanhf(s[sub][j] * cap_inv);
     }
     // ---- mask, running max, weights
     if (masked) {
@@ -549,7 +556,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, float scale,
-    int window, int cus, float* __restrict__ partial, int chunk_tiles, int max_chunks) {
+    int window, float softcap, int cus, float* __restrict__ partial, int chunk_tiles, int max_chunks) {
   static_assert(!(SPLIT && CHUNKED), "a chunk is taken by a workgroup of eight waves");
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef __attribute__((address_space(1))) const void* global_ptr;
@@ -591,7 +598,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = first_pos + tile_off;
-  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int begin = first_visible(tile_first_pos, window);
   const int end = tile_first_pos + tile_cols;
   const int first_tile = begin & ~(PT_KV - 1);
   const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
@@ -602,15 +609,15 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   const int c = q_off + lr;
   const bool col_ok = c < count;
   const int col_pos = col_ok ? first_pos + c : -1;
-  const int col_lo = (window > 0 && col_pos + 1 > window) ? col_pos + 1 - window : 0;
+  const int col_lo = first_visible(col_pos, window);
   bf16x8 qf[KS];
   load_q(col_ok ? q + (size_t)(tok0 + c) * q_stride + (size_t)h * hd : nullptr, hd, qf);
   const int wave_cols = max(0, min(16, count - q_off));
   const int wave_end = wave_cols > 0 ? first_pos + q_off + wave_cols : 0;
   const int wave_first = first_pos + q_off;
-  const int wave_begin = (window > 0 && wave_first + 1 > window) ? wave_first + 1 - window : 0;
+  const int wave_begin = first_visible(wave_first, window);
   const int wave_last = wave_end - 1;
-  const int wave_lo_max = (window > 0 && wave_last + 1 > window) ? wave_last + 1 - window : 0;
+  const int wave_lo_max = first_visible(wave_last, window);
 
   f32x4 o[DT];
   float m = -INFINITY, l = 0.f;
@@ -675,6 +682,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     v_at[st] = (unsigned)(PD_KBYTES + lr * 128 + (((st * 4 + lg) ^ (lr & 7)) * 16));
 
   const float c2 = scale * 1.44269504088896341f;
+  const float cap_raw = softcap > 0.f ? softcap / scale : 0.f, cap_inv = softcap > 0.f ? scale / softcap : 0.f;
   auto tile_body = [&](bool masked, int p0, const unsigned char* base) {
     // ---- scores: tile sub = 2 st + t holds positions p0 + 32 st + 8 g + 4 t + j in register j of lane group g
     f32x4 s[4];
@@ -687,6 +695,12 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
       }
       s[sub] = acc;
+    }
+    if (softcap > 0.f) {   // raw scores whose product with the scale is the capped score
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s[sub][j] = cap_raw * tanhf(s[sub][j] * cap_inv);
     }
     if (masked) {
 #pragma unroll
@@ -815,14 +829,14 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
                                                                  const int* __restrict__ tiles,
                                                                  const int* __restrict__ entry_start,
                                                                  const int* __restrict__ entry_first_pos, int heads,
-                                                                 float scale, int window, int chunk_tiles, int max_chunks) {
+                                                                 float scale, int window, float softcap, int chunk_tiles, int max_chunks) {
   constexpr int hd = HDP, QUADS = HDP / 4, AHEAD = 4;
   const int tile = blockIdx.x, h = blockIdx.y;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
   const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = entry_first_pos[entry] + tile_off;
-  const int begin = (window > 0 && tile_first_pos + 1 > window) ? tile_first_pos + 1 - window : 0;
+  const int begin = first_visible(tile_first_pos, window);
   const int end = tile_first_pos + tile_cols;
   const int first_tile = begin & ~(PT_KV - 1);
   const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
@@ -889,7 +903,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, __bf16* __restrict__ out,
     const int* __restrict__ entries, const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, int chunk, int head_blocks, int dense) {
+    float scale, int window, float softcap, int chunk, int head_blocks, int dense) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
   const int wave = JOINED ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   const int chunk_index = JOINED ? wave : blockIdx.z, chunks = JOINED ? (int)(blockDim.x >> 6) : (int)gridDim.z;
@@ -905,7 +919,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
   if (REGS && window == 0)
     early_pages = block_table[(size_t)entry * table_width + min(ps.page(chunk_index * chunk) + lane, table_width - 1)];
   const int pos = entry_first_pos[entry];
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = first_visible(pos, window);
   const int begin = max(lo, chunk_index * chunk), end = min(pos + 1, (chunk_index + 1) * chunk);
   const int head_in_group = hb * 16 + lr;
   const bool col_ok = head_in_group < group;
@@ -932,7 +946,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
       const int index = cv.page0 + lane;
       if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
     }
-    attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, o, m, l);
+    attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, softcap, o, m, l);
     l = sum_of_column(l);
   }
   if constexpr (JOINED) {
@@ -1067,15 +1081,15 @@ extern "C" int vk_attn_bf16_hdp() { return HDP; }
 // chunk_tiles > 0 (with the kernel that loads straight into LDS; ignored otherwise): a tile's steps of 64 positions
 // are cut into chunks of that many, a workgroup each, of which no tile has more than `max_chunks`; `partial` holds
 // num_tiles * heads * max_chunks * 128 * (padded head width + 4) floats.
-extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+extern "C" int vk_attn_bf16_prefill_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
-                                    int block_size, int heads, int kv_heads, int hd, float scale, int window,
+                                    int block_size, int heads, int kv_heads, int hd, float scale, int window, float softcap,
                                     int split, float* partial, long long partial_floats, int chunk_tiles,
                                     int max_chunks, void* stream) {
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
-      heads % kv_heads || (q_stride & 7) || window < 0)
+      heads % kv_heads || (q_stride & 7))
     return VK_UNSUPPORTED_SIZE;
   constexpr int lds_bytes = (PT_KV * PT_KROW + HDP * PT_VROW) * (int)sizeof(__bf16);
   // page sizes that are powers of two dividing 64 take the kernel with fixed piece addresses
@@ -1112,11 +1126,11 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     }
     chunked<<<num_tiles * heads * max_chunks, PT_THREADS, 2 * PD_STAGE, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus, partial,
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, cus, partial,
         chunk_tiles, max_chunks);
     VK_LAUNCH_CHECK();
     attn_prefill_merge_kernel<<<dim3(num_tiles, heads, PT_TOKENS * (HDP / 4) / 256), 256, 0, (hipStream_t)stream>>>(
-        partial, (__bf16*)out, tiles, entry_start, entry_first_pos, heads, scale, window, chunk_tiles, max_chunks);
+        partial, (__bf16*)out, tiles, entry_start, entry_first_pos, heads, scale, window, softcap, chunk_tiles, max_chunks);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -1135,14 +1149,14 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
     }
     direct<<<num_tiles * heads, halves ? 2 * PT_THREADS : PT_THREADS, direct_lds, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, cus, nullptr, 0, 1);
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, cus, nullptr, 0, 1);
     VK_LAUNCH_CHECK();
     return 0;
   }
 #endif
   kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, cus);
+      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, cus);
   VK_LAUNCH_CHECK();
   return 0;
 }
@@ -1151,14 +1165,14 @@ extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const voi
 // num_entries * heads * chunks * (hd + 2) floats. `chunks` must cover the longest visible range:
 // chunks * chunk >= longest position + 1. `join` nonzero: one workgroup of `chunks` waves (at most 8) per entry and
 // key head merges its chunks itself and writes `out`; `partial` is not used and may be null.
-extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                    void* out, float* partial, const int* entries, int num_entries,
                                    const int* entry_start, const int* entry_first_pos, const int* block_table,
                                    int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                   int window, int chunk, int chunks, int dense, int join, void* stream) {
+                                   int window, float softcap, int chunk, int chunks, int dense, int join, void* stream) {
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
-      heads % kv_heads || (q_stride & 7) || window < 0 || chunk < 32 || (chunk & 31) || chunks <= 0 ||
+      heads % kv_heads || (q_stride & 7) || chunk < 32 || (chunk & 31) || chunks <= 0 ||
       chunks > MAX_CHUNKS)
     return VK_UNSUPPORTED_SIZE;
   if (join && chunks > JOINED_WAVES) return VK_UNSUPPORTED_SIZE;
@@ -1180,7 +1194,7 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
     }
     kernel<<<dim3(num_entries, kv_heads * head_blocks), chunks * 64, lds_bytes, s>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, nullptr, (__bf16*)out, entries,
-        entry_start, entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, chunk,
+        entry_start, entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, chunk,
         head_blocks, dense);
     VK_LAUNCH_CHECK();
     return 0;
@@ -1189,10 +1203,32 @@ extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void
   auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true, false> : attn_decode_kernel<false, false>;
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
                              (__bf16*)out, entries, entry_start, entry_first_pos, block_table, table_width, block_size,
-                             heads, kv_heads, hd, scale, window, chunk, head_blocks, dense);
+                             heads, kv_heads, hd, scale, window, softcap, chunk, head_blocks, dense);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
   attn_combine_kernel<<<cgrid, CB_THREADS, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+// The same two without a cap on the scores.
+extern "C" int vk_attn_bf16_prefill(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                    void* out, const int* tiles, int num_tiles, const int* entry_start,
+                                    const int* entry_first_pos, const int* block_table, int table_width,
+                                    int block_size, int heads, int kv_heads, int hd, float scale, int window,
+                                    int split, float* partial, long long partial_floats, int chunk_tiles,
+                                    int max_chunks, void* stream) {
+  return vk_attn_bf16_prefill_capped(q, q_stride, k_cache, v_cache, out, tiles, num_tiles, entry_start,
+                                     entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale,
+                                     window, 0.f, split, partial, partial_floats, chunk_tiles, max_chunks, stream);
+}
+
+extern "C" int vk_attn_bf16_decode(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                   void* out, float* partial, const int* entries, int num_entries,
+                                   const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                   int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                   int window, int chunk, int chunks, int dense, int join, void* stream) {
+  return vk_attn_bf16_decode_capped(q, q_stride, k_cache, v_cache, out, partial, entries, num_entries, entry_start,
+                                    entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale,
+                                    window, 0.f, chunk, chunks, dense, join, stream);
 }

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ entry_of_token,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, const int* __restrict__ skip_single_of) {
+    float scale, int window, float softcap, const int* __restrict__ skip_single_of) {
   // skip_single_of (entry_start, or null): tokens of entries that hold one token are left to the decode kernel
   if (skip_single_of) {
     const int e = entry_of_token[blockIdx.x];
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
   const int kvh = h / (heads / kv_heads);
   const int pos = positions[t];
   const int hi = pos + 1;
-  const int lo = (window > 0 && hi > window) ? hi - window : 0;
+  const int lo = first_visible(pos, window);
   const int* table = block_table + (size_t)entry_of_token[t] * table_width;
 
   for (int d = tid; d < hd; d += THREADS) q_s[d] = to_float<T>(q[(size_t)t * q_stride + (size_t)h * hd + d]);
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
       const T* k_row = k_cache + (((size_t)page * kv_heads + kvh) * block_size + (p % block_size)) * hd;
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float<T>(k_row[d]), dot);
-      s = dot * scale;
+      s = capped(dot * scale, softcap);
     }
     const float tile_max = block_max(s, red);
     const float m_new = fmaxf(m, tile_max);
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
     const float* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, int head_blocks) {
+    float scale, int window, float softcap, int head_blocks) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   __shared__ float sw[4][HB][DEC_WAVE];                 // a wave's scores, then its weights
   __shared__ float merge_o[4][HB][MAX_HD];              // the waves' weighted sums
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int group = heads / kv_heads;
   const int token = entry_start[entry], pos = entry_first_pos[entry];
-  const int lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int lo = first_visible(pos, window);
   const int chunk_begin = blockIdx.z * DEC_CHUNK;
   const int first_head = kvh * group + hb * HB;                       // of this block of heads
   const int block_heads = min(HB, group - hb * HB);
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
         for (int h = 0; h < HB; ++h) {
 #pragma unroll
           for (int off = 1; off < 16; off <<= 1) dot[h] += __shfl_xor(dot[h], off, WAVE);
-          if (c == 0) sw[wave][h][(it0 + b) * 4 + ps] = (p >= lo && p <= pos) ? dot[h] * scale : -INFINITY;
+          if (c == 0) sw[wave][h][(it0 + b) * 4 + ps] = (p >= lo && p <= pos) ? capped(dot[h] * scale, softcap) : -INFINITY;
         }
       }
     }
@@ -346,7 +346,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const float* __restrict__ q, long long q_stride, const float* __restrict__ k_cache,
     const float* __restrict__ v_cache, float* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, const int* __restrict__ block_table,
-    int table_width, int block_size, int heads, int kv_heads, float scale, int window, int tile_tokens) {
+    int table_width, int block_size, int heads, int kv_heads, float scale, int window, float softcap, int tile_tokens) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   constexpr int HD = 16 * DPT, QROW = HD + 4, VROW = PF_TILE + 4;
   extern __shared__ __attribute__((aligned(16))) float pf_lds[];
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
 #pragma unroll
     for (int j = 0; j < DPT; ++j) o[i][j] = 0.f;
   }
-  const int lowest = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;   // the first token's first position
+  const int lowest = first_visible(pos0, window);   // the first token's first position
   for (int kv0 = lowest / PF_TILE * PF_TILE; kv0 <= last_pos; kv0 += PF_TILE) {
     __syncthreads();   // the tile before has been read
     for (int i = tid; i < PF_TILE * (HD / 4); i += 256) {
@@ -439,13 +439,13 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int qpos = pos0 + 4 * ty + i;
-      const int first = (window > 0 && qpos + 1 > window) ? qpos + 1 - window : 0;
+      const int first = first_visible(qpos, window);
       float best = -INFINITY;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int p = kv0 + tx + 16 * j;
         const bool sees = 4 * ty + i < rows && p <= qpos && p >= first;
-        s[i][j] = sees ? s[i][j] * scale : -INFINITY;
+        s[i][j] = sees ? capped(s[i][j] * scale, softcap) : -INFINITY;
         best = fmaxf(best, s[i][j]);
       }
 #pragma unroll
@@ -503,7 +503,7 @@ template <int DPT>
 int launch_prefill_f32(dim3 grid, hipStream_t s, const float* q, long long q_stride, const float* k_cache,
                        const float* v_cache, float* out, const int* tiles, const int* entry_start,
                        const int* entry_first_pos, const int* block_table, int table_width, int block_size, int heads,
-                       int kv_heads, float scale, int window, int tile_tokens) {
+                       int kv_heads, float scale, int window, float softcap, int tile_tokens) {
   constexpr int HD = 16 * DPT;
   constexpr int lds_bytes = (2 * PF_TILE * (HD + 4) + HD * (PF_TILE + 4) + PF_TILE * (PF_TILE + 4)) * 4;
   static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KB of LDS");
@@ -516,7 +516,7 @@ int launch_prefill_f32(dim3 grid, hipStream_t s, const float* q, long long q_str
   }
   attn_prefill_f32_kernel<DPT><<<grid, 256, lds_bytes, s>>>(q, q_stride, k_cache, v_cache, out, tiles, entry_start,
                                                             entry_first_pos, block_table, table_width, block_size,
-                                                            heads, kv_heads, scale, window, tile_tokens);
+                                                            heads, kv_heads, scale, window, softcap, tile_tokens);
   return 0;
 }
 
@@ -524,22 +524,21 @@ template <int HB, int QC>
 void launch_decode_f32(dim3 grid, hipStream_t s, const float* q, long long q_stride, const float* k_cache,
                        const float* v_cache, float* partial, const int* entries, const int* entry_start,
                        const int* entry_first_pos, const int* block_table, int table_width, int block_size, int heads,
-                       int kv_heads, int hd, float scale, int window, int head_blocks) {
+                       int kv_heads, int hd, float scale, int window, float softcap, int head_blocks) {
   attn_decode_f32_kernel<HB, QC><<<grid, 256, 0, s>>>(q, q_stride, k_cache, v_cache, partial, entries, entry_start,
                                                       entry_first_pos, block_table, table_width, block_size, heads,
-                                                      kv_heads, hd, scale, window, head_blocks);
+                                                      kv_heads, hd, scale, window, softcap, head_blocks);
 }
 }  // namespace
 
-extern "C" int vk_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+extern "C" int vk_attn_generic_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                void* out, int dtype, const int* positions, const int* entry_of_token,
                                const int* block_table, int table_width, int block_size, int num_tokens, int heads,
-                               int kv_heads, int hd, float scale, int window, const int* skip_single_of,
+                               int kv_heads, int hd, float scale, int window, float softcap, const int* skip_single_of,
                                void* stream) {
   if (num_tokens <= 0) return 0;
   if (hd <= 0 || hd > MAX_HD) return VK_UNSUPPORTED_SIZE;
-  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || block_size <= 0 || table_width <= 0 ||
-      window < 0)
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || block_size <= 0 || table_width <= 0)
     return VK_BAD_ARGUMENT;
   dim3 grid(num_tokens, heads);
   hipStream_t s = (hipStream_t)stream;
@@ -547,12 +546,12 @@ extern "C" int vk_attn_generic(const void* q, long long q_stride, const void* k_
     attn_generic_kernel<float><<<grid, THREADS, 0, s>>>((const float*)q, q_stride, (const float*)k_cache,
                                                         (const float*)v_cache, (float*)out, positions,
                                                         entry_of_token, block_table, table_width, block_size,
-                                                        heads, kv_heads, hd, scale, window, skip_single_of);
+                                                        heads, kv_heads, hd, scale, window, softcap, skip_single_of);
   else if (dtype == DT_BF16)
     attn_generic_kernel<bf16_t><<<grid, THREADS, 0, s>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                                          (const bf16_t*)v_cache, (bf16_t*)out, positions,
                                                          entry_of_token, block_table, table_width, block_size,
-                                                         heads, kv_heads, hd, scale, window, skip_single_of);
+                                                         heads, kv_heads, hd, scale, window, softcap, skip_single_of);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
@@ -565,14 +564,14 @@ extern "C" int vk_attn_decode_f32_chunk() { return DEC_CHUNK; }
 
 // Attention of the single-token entries listed in `entries` in 32-bit: float q, cache and out. partial: at least
 // num_entries * heads * chunks * (hd + 2) floats; chunks * 256 >= longest position + 1.
-extern "C" int vk_attn_decode_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+extern "C" int vk_attn_decode_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
                                   float* out, float* partial, const int* entries, int num_entries,
                                   const int* entry_start, const int* entry_first_pos, const int* block_table,
                                   int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                  int window, int chunks, void* stream) {
+                                  int window, float softcap, int chunks, void* stream) {
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > MAX_HD || (hd & 3) || block_size <= 0 || (block_size & 3) || (q_stride & 3)) return VK_UNSUPPORTED_SIZE;
-  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || table_width <= 0 || window < 0 || chunks <= 0 ||
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || table_width <= 0 || chunks <= 0 ||
       chunks > 65535)
     return VK_BAD_ARGUMENT;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15)) return VK_BAD_ARGUMENT;
@@ -588,7 +587,7 @@ extern "C" int vk_attn_decode_f32(const float* q, long long q_stride, const floa
   dim3 grid(num_entries, kv_heads * head_blocks, chunks);
 #define VK_DEC(HBV, QCV)                                                                                          \
   launch_decode_f32<HBV, QCV>(grid, s, q, q_stride, k_cache, v_cache, partial, entries, entry_start, entry_first_pos, \
-                              block_table, table_width, block_size, heads, kv_heads, hd, scale, window, head_blocks)
+                              block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, head_blocks)
   if (qc == 1) {
     switch (hb) { case 1: VK_DEC(1, 1); break; case 2: VK_DEC(2, 1); break; case 4: VK_DEC(4, 1); break; default: VK_DEC(8, 1); }
   } else if (qc == 2) {
@@ -606,13 +605,13 @@ extern "C" int vk_attn_decode_f32(const float* q, long long q_stride, const floa
 // Attention of the step's prompt portions in 32-bit: float q, cache and out. tiles: pairs (entry, first token of the
 // tile within the entry), `tile_tokens` tokens a tile (a multiple of 64), as vk_attn_bf16_prefill takes them. Head
 // widths that are multiples of 16 up to 128, pages of a multiple of 4 positions.
-extern "C" int vk_attn_prefill_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+extern "C" int vk_attn_prefill_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
                                    float* out, const int* tiles, int num_tiles, int tile_tokens, const int* entry_start,
                                    const int* entry_first_pos, const int* block_table, int table_width, int block_size,
-                                   int heads, int kv_heads, int hd, float scale, int window, void* stream) {
+                                   int heads, int kv_heads, int hd, float scale, int window, float softcap, void* stream) {
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > 128 || (hd & 15) || block_size <= 0 || (block_size & 3) || (q_stride & 3)) return VK_UNSUPPORTED_SIZE;
-  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || table_width <= 0 || window < 0 ||
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || table_width <= 0 ||
       tile_tokens <= 0 || tile_tokens % PF_TILE)
     return VK_BAD_ARGUMENT;
   if (((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15)) return VK_BAD_ARGUMENT;
@@ -624,11 +623,41 @@ extern "C" int vk_attn_prefill_f32(const float* q, long long q_stride, const flo
 #define VK_PF(DPTV)                                                                                                  \
   case DPTV:                                                                                                         \
     status = launch_prefill_f32<DPTV>(grid, s, q, q_stride, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, \
-                                      block_table, table_width, block_size, heads, kv_heads, scale, window, tile_tokens); \
+                                      block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, tile_tokens); \
     break;
   switch (hd / 16) { VK_PF(1) VK_PF(2) VK_PF(3) VK_PF(4) VK_PF(5) VK_PF(6) VK_PF(7) VK_PF(8) }
 #undef VK_PF
   if (status != 0) return status;
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+// The same three without a cap on the scores.
+extern "C" int vk_attn_generic(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                               void* out, int dtype, const int* positions, const int* entry_of_token,
+                               const int* block_table, int table_width, int block_size, int num_tokens, int heads,
+                               int kv_heads, int hd, float scale, int window, const int* skip_single_of,
+                               void* stream) {
+  return vk_attn_generic_capped(q, q_stride, k_cache, v_cache, out, dtype, positions, entry_of_token, block_table,
+                                table_width, block_size, num_tokens, heads, kv_heads, hd, scale, window, 0.f,
+                                skip_single_of, stream);
+}
+
+extern "C" int vk_attn_decode_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                  float* out, float* partial, const int* entries, int num_entries,
+                                  const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                  int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                  int window, int chunks, void* stream) {
+  return vk_attn_decode_f32_capped(q, q_stride, k_cache, v_cache, out, partial, entries, num_entries, entry_start,
+                                   entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale,
+                                   window, 0.f, chunks, stream);
+}
+
+extern "C" int vk_attn_prefill_f32(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                   float* out, const int* tiles, int num_tiles, int tile_tokens, const int* entry_start,
+                                   const int* entry_first_pos, const int* block_table, int table_width, int block_size,
+                                   int heads, int kv_heads, int hd, float scale, int window, void* stream) {
+  return vk_attn_prefill_f32_capped(q, q_stride, k_cache, v_cache, out, tiles, num_tiles, tile_tokens, entry_start,
+                                    entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale,
+                                    window, 0.f, stream);
 }

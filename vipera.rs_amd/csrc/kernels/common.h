@@ -56,6 +56,16 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return best;
 }
 
+// Which positions a token at `pos` attends to, [first_visible, pos]: everything before it (window 0), the last
+// `window` positions (window > 0), or the positions of its own block of `-window` consecutive positions, counted
+// from position 0 of the sequence (window < 0).  It never falls as `pos` grows.
+__device__ __forceinline__ int first_visible(int pos, int window) {
+  return window > 0 ? max(pos + 1 - window, 0) : window < 0 ? pos - pos % (-window) : 0;
+}
+
+// A score bounded by a soft cap: cap * tanh(s / cap); cap 0: the score as it is.
+__device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
+
 // Status codes of the extern "C" launchers: 0 ok, a positive hipError_t, or one of these.
 constexpr int VK_BAD_ARGUMENT = -1;
 constexpr int VK_UNSUPPORTED_SIZE = -2;

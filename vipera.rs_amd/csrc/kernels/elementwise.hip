@@ -513,3 +513,197 @@ extern "C" int vk_scale(float* x, float factor, long long count, void* stream) {
   VK_LAUNCH_CHECK();
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------------
+// A norm behind a sublayer: residual[r, :] += y[r, :] / sqrt(mean(y[r, :]^2) + eps) * weight, all 32-bit.
+// One workgroup per row; the sum of squares in the order of `rmsnorm_kernel`'s general path.
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restrict__ y, const float* __restrict__ weight,
+                                                          float* __restrict__ residual, int width, float eps) {
+  __shared__ float scratch[16];
+  const float* src = y + (size_t)blockIdx.x * width;
+  float* dst = residual + (size_t)blockIdx.x * width;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = src[i];
+    sum += v * v;
+  }
+  sum = block_sum(sum, scratch);
+  const float inv = 1.0f / sqrtf(sum / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += 256) dst[i] += src[i] * inv * weight[i];
+}
+
+extern "C" int vk_rmsnorm_add(const float* y, const float* weight, float* residual, int num_rows, int width, float eps,
+                              void* stream) {
+  if (num_rows <= 0) return 0;
+  if (width <= 0) return VK_BAD_ARGUMENT;
+  rmsnorm_add_kernel<<<num_rows, 256, 0, (hipStream_t)stream>>>(y, weight, residual, width, eps);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// out (+)= a * x + b * y, elementwise, 32-bit.
+__global__ void axpby_kernel(const float* __restrict__ x, float a, const float* __restrict__ y, float b,
+                             float* __restrict__ out, long long count, int accumulate) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  const float v = fmaf(a, x[i], b * y[i]);
+  out[i] = accumulate ? out[i] + v : v;
+}
+
+extern "C" int vk_axpby(const float* x, float a, const float* y, float b, float* out, long long count, int accumulate,
+                        void* stream) {
+  if (count <= 0) return 0;
+  axpby_kernel<<<(unsigned)((count + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, a, y, b, out, count, accumulate);
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// out[r, c] = act(in[r, c]) (* mul[r, c]); rows of `in` and `mul` may be strided.
+//   act 0: as it is (a change of type), 1: relu squared, 2: silu, 3: gelu (tanh form), 4: sigmoid
+__device__ __forceinline__ float apply_act(float z, int act) {
+  switch (act) {
+    case 1: { const float r = fmaxf(z, 0.f); return r * r; }
+    case 2: return z / (1.0f + expf(-z));
+    case 3: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    case 4: return 1.0f / (1.0f + expf(-z));
+    default: return z;
+  }
+}
+
+template <typename TI, typename TM, typename TO>
+__global__ void activation_kernel(const TI* __restrict__ in, long long ldi, const TM* __restrict__ mul, long long ldm,
+                                  TO* __restrict__ out, int width, long long total, int act) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long r = idx / width;
+  const int c = (int)(idx % width);
+  float v = apply_act(to_float<TI>(in[r * ldi + c]), act);
+  if (mul) v *= to_float<TM>(mul[r * ldm + c]);
+  out[idx] = from_float<TO>(v);
+}
+
+extern "C" int vk_activation(const void* in, int in_dtype, long long ldi, const void* mul, int mul_dtype, long long ldm,
+                             void* out, int out_dtype, int num_rows, int width, int act, void* stream) {
+  if (num_rows <= 0) return 0;
+  if (width <= 0 || act < 0 || act > 4) return VK_BAD_ARGUMENT;
+  const long long total = (long long)num_rows * width;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (mul == nullptr) mul_dtype = DT_F32;
+#define VK_ACT(TI, TM, TO)                                                                                          \
+  activation_kernel<TI, TM, TO><<<blocks, 256, 0, s>>>((const TI*)in, ldi, (const TM*)mul, ldm, (TO*)out, width, total, act)
+#define VK_ACT_O(TI, TM)                                \
+  if (out_dtype == DT_F32) VK_ACT(TI, TM, float);       \
+  else if (out_dtype == DT_BF16) VK_ACT(TI, TM, bf16_t); \
+  else return VK_BAD_ARGUMENT
+#define VK_ACT_M(TI)                                      \
+  if (mul_dtype == DT_F32) { VK_ACT_O(TI, float); }       \
+  else if (mul_dtype == DT_BF16) { VK_ACT_O(TI, bf16_t); } \
+  else return VK_BAD_ARGUMENT
+  if (in_dtype == DT_F32) { VK_ACT_M(float); }
+  else if (in_dtype == DT_BF16) { VK_ACT_M(bf16_t); }
+  else return VK_BAD_ARGUMENT;
+#undef VK_ACT_M
+#undef VK_ACT_O
+#undef VK_ACT
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Queries and keys normed over the whole projection, and all three laid out as the attention kernels read them.
+//   proj [T, ldp] 32-bit: q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim) from column 0 on
+//   q <- q / rms(q) * q_weight over all heads * dim numbers at once, k likewise (weights may be null: no norm)
+//   qkv  [T, (heads + 2 kv_heads) * W]: every head padded with zeros to W >= max(dim, vdim)
+// One workgroup per token.
+template <typename TO>
+__global__ __launch_bounds__(256) void whole_norm_pack_kernel(const float* __restrict__ proj, long long ldp,
+                                                              const float* __restrict__ q_weight,
+                                                              const float* __restrict__ k_weight, float eps, int heads,
+                                                              int kv_heads, int dim, int vdim, int W,
+                                                              TO* __restrict__ qkv) {
+  __shared__ float scratch[16];
+  const float* src = proj + (size_t)blockIdx.x * ldp;
+  TO* dst = qkv + (size_t)blockIdx.x * (heads + 2 * kv_heads) * W;
+  const int qn = heads * dim, kn = kv_heads * dim, vn = kv_heads * vdim;
+  float qs = 0.f, ks = 0.f;
+  if (q_weight)
+    for (int i = threadIdx.x; i < qn; i += 256) qs += src[i] * src[i];
+  if (k_weight)
+    for (int i = threadIdx.x; i < kn; i += 256) ks += src[qn + i] * src[qn + i];
+  qs = block_sum(qs, scratch);
+  ks = block_sum(ks, scratch);
+  const float q_inv = 1.0f / sqrtf(qs / (float)qn + eps), k_inv = 1.0f / sqrtf(ks / (float)kn + eps);
+  for (int i = threadIdx.x; i < heads * W; i += 256) {
+    const int h = i / W, d = i % W;
+    float v = 0.f;
+    if (d < dim) {
+      v = src[h * dim + d];
+      if (q_weight) v = v * q_inv * q_weight[h * dim + d];
+    }
+    dst[i] = from_float<TO>(v);
+  }
+  for (int i = threadIdx.x; i < kv_heads * W; i += 256) {
+    const int h = i / W, d = i % W;
+    float v = 0.f;
+    if (d < dim) {
+      v = src[qn + h * dim + d];
+      if (k_weight) v = v * k_inv * k_weight[h * dim + d];
+    }
+    dst[heads * W + i] = from_float<TO>(v);
+    dst[(heads + kv_heads) * W + i] = from_float<TO>(d < vdim ? src[qn + kn + h * vdim + d] : 0.f);
+  }
+  (void)vn;
+}
+
+extern "C" int vk_whole_norm_pack(const float* proj, long long ldp, const float* q_weight, const float* k_weight,
+                                  float eps, int num_tokens, int heads, int kv_heads, int dim, int vdim, int W, void* qkv,
+                                  int dtype, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || dim < 1 || vdim < 1 || W < dim || W < vdim) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    whole_norm_pack_kernel<float><<<num_tokens, 256, 0, s>>>(proj, ldp, q_weight, k_weight, eps, heads, kv_heads, dim,
+                                                             vdim, W, (float*)qkv);
+  else if (dtype == DT_BF16)
+    whole_norm_pack_kernel<bf16_t><<<num_tokens, 256, 0, s>>>(proj, ldp, q_weight, k_weight, eps, heads, kv_heads, dim,
+                                                              vdim, W, (bf16_t*)qkv);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+// The attention's output taken out of its padded heads and gated:
+//   out[t, h * vdim + d] = attn[t, h * W + d] * gate(g[t, h * vdim + d]);  gate_act as in vk_activation, g null: none
+template <typename T>
+__global__ void head_unpack_gate_kernel(const T* __restrict__ attn, const float* __restrict__ g, long long ldg,
+                                        int gate_act, int heads, int vdim, int W, long long total, T* __restrict__ out) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int width = heads * vdim;
+  const long long t = idx / width;
+  const int c = (int)(idx % width), h = c / vdim, d = c % vdim;
+  float v = to_float<T>(attn[(t * heads + h) * W + d]);
+  if (g) v *= apply_act(g[t * ldg + c], gate_act);
+  out[idx] = from_float<T>(v);
+}
+
+extern "C" int vk_head_unpack_gate(const void* attn, int dtype, const float* g, long long ldg, int gate_act,
+                                   int num_tokens, int heads, int vdim, int W, void* out, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads < 1 || vdim < 1 || W < vdim || gate_act < 0 || gate_act > 4) return VK_BAD_ARGUMENT;
+  const long long total = (long long)num_tokens * heads * vdim;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DT_F32)
+    head_unpack_gate_kernel<float><<<blocks, 256, 0, s>>>((const float*)attn, g, ldg, gate_act, heads, vdim, W, total,
+                                                          (float*)out);
+  else if (dtype == DT_BF16)
+    head_unpack_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>((const bf16_t*)attn, g, ldg, gate_act, heads, vdim, W, total,
+                                                           (bf16_t*)out);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}

@@ -15,11 +15,51 @@ constexpr int MOE_TILE = 64;      // places per tile of the 32-bit products; the
 // ---------------------------------------------------------------------------------------------
 // One wave per token: the `top` largest of E logits (the lowest id wins a tie), and the softmax over those.
 // Lane l looks after experts l, l + 64, ...; a bit per expert of its own says which are taken (E <= 4096).
+//
+// `groups` > 1: the experts form that many equal groups of neighbours, a group's score is its largest logit, and
+// only experts of the `keep` best groups (the lowest group among equals) can be chosen.  `all_scores`: the weights are
+// the chosen experts' shares of the softmax over all E logits, which do not add up to one.
+struct Routing {
+  int groups, keep, all_scores;
+};
+
 __device__ __forceinline__ void route_token(const float* __restrict__ logits, int experts, int top, int t, int lane,
-                                            int* __restrict__ ids, float* __restrict__ weights) {
+                                            int* __restrict__ ids, float* __restrict__ weights,
+                                            Routing how = Routing{1, 1, 0}) {
   constexpr int NONE = 0x7fffffff;
   const float* z = logits + (long long)t * experts;
   unsigned long long taken = 0;
+  if (how.groups > 1 && how.keep < how.groups) {
+    // lane g keeps group g's score (at most 64 groups); the experts of the groups that lose count as taken
+    const int size = experts / how.groups;
+    float score = -INFINITY;
+    if (lane < how.groups)
+      for (int e = lane * size; e < (lane + 1) * size; ++e) score = fmaxf(score, z[e]);
+    unsigned long long kept = 0;
+    for (int j = 0; j < how.keep; ++j) {
+      float best = (lane < how.groups && !((kept >> lane) & 1ull)) ? score : -INFINITY;
+      int arg = (lane < how.groups && !((kept >> lane) & 1ull)) ? lane : NONE;
+      for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, WAVE);
+        const int oa = __shfl_xor(arg, off, WAVE);
+        if (oa != NONE && (arg == NONE || ob > best || (ob == best && oa < arg))) {
+          best = ob;
+          arg = oa;
+        }
+      }
+      if (arg != NONE) kept |= 1ull << arg;
+    }
+    for (int e = lane, i = 0; e < experts; e += WAVE, ++i)
+      if (!((kept >> (e / size)) & 1ull)) taken |= 1ull << i;
+  }
+  float whole_max = -INFINITY, whole_sum = 1.f;
+  if (how.all_scores) {
+    for (int e = lane; e < experts; e += WAVE) whole_max = fmaxf(whole_max, z[e]);
+    whole_max = wave_max(whole_max);
+    float part = 0.f;
+    for (int e = lane; e < experts; e += WAVE) part += expf(z[e] - whole_max);
+    whole_sum = wave_sum(part);
+  }
   float first = 0.f, sum = 0.f, mine = 0.f;      // lane j keeps the weight of choice j
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
@@ -42,19 +82,19 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     }
     if ((arg & (WAVE - 1)) == lane) taken |= 1ull << (arg / WAVE);
     if (j == 0) first = best;
-    const float p = expf(best - first);
+    const float p = how.all_scores ? expf(best - whole_max) : expf(best - first);
     sum += p;
     if (lane == j) mine = p;
     if (lane == 0) ids[(long long)t * top + j] = arg;
   }
-  if (lane < top) weights[(long long)t * top + lane] = mine / sum;
+  if (lane < top) weights[(long long)t * top + lane] = mine / (how.all_scores ? whole_sum : sum);
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
                                                         int num_tokens, int* __restrict__ ids,
-                                                        float* __restrict__ weights) {
+                                                        float* __restrict__ weights, Routing how) {
   const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-  if (t < num_tokens) route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights);
+  if (t < num_tokens) route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights, how);
 }
 
 // One workgroup: counts per expert, offsets, the pairs' places, and the list of tiles.
@@ -65,13 +105,13 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const float* __restrict
                                                          float* __restrict__ weights, int* __restrict__ ids, int pairs,
                                                          int experts, int tile_rows, int* __restrict__ offsets,
                                                          int* __restrict__ order, int* __restrict__ tiles,
-                                                         int* __restrict__ num_tiles) {
+                                                         int* __restrict__ num_tiles, Routing how) {
   extern __shared__ int shared[];      // counts [E], cursor [E]
   int* counts = shared;
   int* cursor = shared + experts;
   if (logits) {
     for (int t = threadIdx.x / WAVE; t < num_tokens; t += blockDim.x / WAVE)
-      route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights);
+      route_token(logits, experts, top, t, threadIdx.x & (WAVE - 1), ids, weights, how);
     __threadfence_block();
     __syncthreads();
   }
@@ -99,8 +139,18 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
-// Gate and up products of a tile with the experts' activation:
-//   g = min(Wg h, limit), u = clamp(Wu h, -limit, limit), y = g * sigmoid(alpha * g) * (u + 1)
+// The experts' activation of a gate sum g and an up sum u.  A finite `limit`: g = min(g, limit),
+// u = clamp(u, -limit, limit), y = g * sigmoid(alpha * g) * (u + 1).  An infinite one: y = g * sigmoid(alpha * g) * u,
+// which with alpha 1 is silu(g) * u.
+__device__ __forceinline__ float expert_act(float g, float u, float limit, float alpha) {
+  if (limit < INFINITY) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+  }
+  return g * (1.0f / (1.0f + expf(-alpha * g))) * u;
+}
+
+// Gate and up products of a tile with the experts' activation (expert_act above).
 // h: [T, width] (row of pair p is p / top); wg, wu: [E, ff, width]; act: [P places, ff].
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ h, long long ldh,
@@ -160,10 +210,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= ff) continue;
-      const float g = fminf(ga[i][j], limit);
-      const float u = fminf(fmaxf(ua[i][j], -limit), limit);
-      const float y = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f);
-      act[(long long)(first + r) * ff + n] = from_float<T>(y);
+      act[(long long)(first + r) * ff + n] = from_float<T>(expert_act(ga[i][j], ua[i][j], limit, alpha));
     }
   }
 }
@@ -260,9 +307,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_mma_kernel(const __bf16* __re
       for (int i = 0; i < 4; ++i) {
         const int col = n0 + wn * 32 + tn * 16 + lg * 4 + i;
         if (col >= ff) continue;
-        const float g = fminf(acc[tn][tm][i], limit);
-        const float u = fminf(fmaxf(acc[tn + 2][tm][i], -limit), limit);
-        act[(long long)(first + r) * ff + col] = (__bf16)(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+        act[(long long)(first + r) * ff + col] = (__bf16)expert_act(acc[tn][tm][i], acc[tn + 2][tm][i], limit, alpha);
       }
   }
 }
@@ -326,9 +371,14 @@ extern "C" int vk_moe_tile_rows(int dtype, int width, int ff, long long ldh) {
   return moe_on_matrix_cores(dtype, width, ff, ldh) ? GT_TILE : MOE_TILE;
 }
 
-extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int tile_rows, int* ids,
-                            float* weights, int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, int num_tokens, int tile_rows, int groups,
+                                    int keep, int all_scores, int* ids, float* weights, int* offsets, int* order,
+                                    int* tiles, int* num_tiles, void* stream) {
   if (tile_rows != MOE_TILE && tile_rows != GT_TILE) return VK_BAD_ARGUMENT;
+  if (groups < 1 || keep < 1 || keep > groups || experts % groups != 0) return VK_BAD_ARGUMENT;
+  if (groups > WAVE) return VK_UNSUPPORTED_SIZE;
+  if (keep < groups && (long long)keep * (experts / groups) < top) return VK_BAD_ARGUMENT;
+  const Routing how{groups, keep, all_scores ? 1 : 0};
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
@@ -337,14 +387,20 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
   if (pairs > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
   const bool together = num_tokens <= 16;     // a wave of the one workgroup for every token
   if (!together) {
-    moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights);
+    moe_route_kernel<<<(num_tokens + 3) / 4, 256, 0, s>>>(logits, experts, top, num_tokens, ids, weights, how);
     VK_LAUNCH_CHECK();
   }
   moe_group_kernel<<<1, 1024, (size_t)experts * 2 * sizeof(int), s>>>(together ? logits : nullptr, top, num_tokens,
                                                                        weights, ids, (int)pairs, experts, tile_rows,
-                                                                       offsets, order, tiles, num_tiles);
+                                                                       offsets, order, tiles, num_tiles, how);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int tile_rows, int* ids,
+                            float* weights, int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+  return vk_moe_route_grouped(logits, experts, top, num_tokens, tile_rows, 1, 1, 0, ids, weights, offsets, order, tiles,
+                              num_tiles, stream);
 }
 
 extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,

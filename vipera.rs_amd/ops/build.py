@@ -36,6 +36,7 @@ MODULES: Dict[str, tuple] = {
     "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h", "kernels/no_alloc.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
     "recurrent": ("hip", ["kernels/recurrent.hip"], ["kernels/common.h"]),
+    "scan": ("hip", ["kernels/scan.hip"], ["kernels/common.h"]),
     "latent": ("hip", ["kernels/latent.hip"], ["kernels/common.h", "kernels/group_tile.h"]),
     "moe": ("hip", ["kernels/moe.hip"], ["kernels/common.h", "kernels/group_tile.h"]),
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],

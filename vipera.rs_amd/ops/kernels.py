@@ -254,8 +254,10 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
 def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                  positions: torch.Tensor, entry_of_token: torch.Tensor, block_table: torch.Tensor,
                  heads: int, kv_heads: int, head_dim: int, scale: float, window: int,
-                 skip_single_of: Optional[torch.Tensor] = None) -> None:
-    """Causal GQA over the paged cache for every token of the step, in 32-bit arithmetic.
+                 skip_single_of: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
+    """Causal GQA over the paged cache for every token of the step, in 32-bit arithmetic.  ``window`` > 0: the last
+    that many positions; < 0: the positions of the token's own block of ``-window`` consecutive positions (counted
+    from position 0); ``softcap`` > 0: scores become ``softcap * tanh(score / softcap)`` (all attention kernels alike).
 
     ``q``: a view ``[tokens, >= heads * head_dim]`` whose row holds the query heads first (the fused
     qkv buffer qualifies); ``out``: ``[tokens, heads * head_dim]``.  ``skip_single_of``: the step's
@@ -275,11 +277,11 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
     if head_dim > ATTENTION_MAX_HEAD_DIM:
         raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of {ATTENTION_MAX_HEAD_DIM}")
-    fn = _fn("attn_generic", "vk_attn_generic",
-             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p, _p])
+    fn = _fn("attn_generic", "vk_attn_generic_capped",
+             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
                _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], k_cache.shape[2], num_tokens, heads,
-               kv_heads, head_dim, float(scale), int(window), _ptr(skip_single_of), _stream()), "attn_generic")
+               kv_heads, head_dim, float(scale), int(window), float(softcap), _ptr(skip_single_of), _stream()), "attn_generic")
 
 
 ATTN_DECODE_F32_CHUNK = 256   # positions of one workgroup of attn_decode_f32 (the kernel's DEC_CHUNK)
@@ -296,7 +298,7 @@ def attn_decode_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: 
 def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                     partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                     entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
-                    head_dim: int, scale: float, window: int, chunks: int) -> None:
+                    head_dim: int, scale: float, window: int, chunks: int, softcap: float = 0.0) -> None:
     """32-bit attention of the single-token entries listed in ``entries``; their positions are split into
     ``chunks`` of :data:`ATTN_DECODE_F32_CHUNK`, which must cover the longest visible range."""
     _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
@@ -314,11 +316,11 @@ def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
     _need(heads % kv_heads == 0 and chunks >= 1, "attention: heads must be a multiple of kv_heads")
-    fn = _fn("attn_generic", "vk_attn_decode_f32",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p])
+    fn = _fn("attn_generic", "vk_attn_decode_f32_capped",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), int(chunks), _stream()), "attn_decode_f32")
+               heads, kv_heads, head_dim, float(scale), int(window), float(softcap), int(chunks), _stream()), "attn_decode_f32")
 
 
 ATTN_PREFILL_F32_MAX_HEAD_DIM = 128   # the K, V and weight tiles of a wider head do not fit a CU's LDS
@@ -335,7 +337,7 @@ def attn_prefill_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim:
 def attn_prefill_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      tiles: torch.Tensor, tile_tokens: int, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                      block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
-                     window: int) -> None:
+                     window: int, softcap: float = 0.0) -> None:
     """32-bit attention of the entries' tiles listed in ``tiles`` (pairs: entry, first token within it; ``tile_tokens``
     tokens a tile, a multiple of 64): 64 tokens of one head a workgroup, the positions in LDS tiles of 64."""
     _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
@@ -351,11 +353,11 @@ def attn_prefill_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
     _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
-    fn = _fn("attn_generic", "vk_attn_prefill_f32",
-             [_p, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _p])
+    fn = _fn("attn_generic", "vk_attn_prefill_f32_capped",
+             [_p, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
                int(tile_tokens), _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1],
-               k_cache.shape[2], heads, kv_heads, head_dim, float(scale), int(window), _stream()), "attn_prefill_f32")
+               k_cache.shape[2], heads, kv_heads, head_dim, float(scale), int(window), float(softcap), _stream()), "attn_prefill_f32")
 
 
 # ----------------------------------------------------------------------------------------------
@@ -727,7 +729,8 @@ ATTN_PREFILL_PARTIAL_ROW_EXTRA = 4   # floats beside the padded head width in a 
 def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                       block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
-                      window: int, split: bool = False, chunk_tiles: int = 0, max_chunks: int = 0) -> None:
+                      window: int, split: bool = False, chunk_tiles: int = 0, max_chunks: int = 0,
+                      softcap: float = 0.0) -> None:
     """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it).
     ``split``: workgroups of sixteen waves that halve a tile's positions between them and merge at the end, where
     the kernel in use has that form (for few tiles of very different lengths); the same result up to rounding.
@@ -752,12 +755,12 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     else:
         chunk_tiles = max_chunks = 0
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_prefill",
-             [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _ll, _i, _i, _p],
+    fn = _fn(module, "vk_attn_bf16_prefill_capped",
+             [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p, _ll, _i, _i, _p],
              key=module + ".prefill")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), num_tiles,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), 1 if split else 0, _ptr(partial),
+               heads, kv_heads, head_dim, float(scale), int(window), float(softcap), 1 if split else 0, _ptr(partial),
                partial.numel() if partial is not None else 0, int(chunk_tiles), int(max_chunks), _stream()),
             "attn_bf16_prefill")
 
@@ -769,7 +772,7 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                      entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
                      head_dim: int, scale: float, window: int, chunk: int, chunks: int, dense: bool = False,
-                     join: bool = False) -> None:
+                     join: bool = False, softcap: float = 0.0) -> None:
     """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``.
     ``dense``: the step holds single-token entries only, so entry i is the i-th of them and holds token i; the
     kernel then need not look either up.  ``join``: one workgroup per entry and key head takes all chunks (at most
@@ -790,11 +793,11 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _need(chunk >= 32 and chunk % 32 == 0 and chunks >= 1, "attention: chunk must be a multiple of 32")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_decode",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _i, _p], key=module + ".decode")
+    fn = _fn(module, "vk_attn_bf16_decode_capped",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _i, _i, _i, _p], key=module + ".decode")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), int(chunk), int(chunks), 1 if dense else 0,
+               heads, kv_heads, head_dim, float(scale), int(window), float(softcap), int(chunk), int(chunks), 1 if dense else 0,
                1 if join else 0, _stream()),
             "attn_bf16_decode")
 
@@ -1141,9 +1144,13 @@ def moe_max_tiles(pairs: int, experts: int, tile_rows: int = 64) -> int:
 
 
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, offsets: torch.Tensor,
-              order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, tile_rows: int = 64) -> None:
+              order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, tile_rows: int = 64,
+              groups: int = 1, keep: int = 1, all_scores: bool = False) -> None:
     """Each token's ``top`` largest router logits (lowest id first among equals) with the softmax over those, and the
-    (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``."""
+    (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``.
+    ``groups`` > 1: the experts form that many equal groups of neighbours and only those of the ``keep`` groups with
+    the largest logits can be chosen.  ``all_scores``: the weights are the chosen experts' shares of the softmax over
+    all experts (they do not add up to one)."""
     _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
     tokens, experts = logits.shape
     _f32(logits, "moe_route: logits")
@@ -1153,16 +1160,19 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
     _need(ids.numel() == tokens * top and weights.numel() == tokens * top and order.numel() == tokens * top
           and offsets.numel() == experts + 1 and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts, tile_rows)
           and num_tiles.numel() == 1 and tile_rows in (64, 128), "moe_route: output sizes")
-    fn = _fn("moe", "vk_moe_route", [_p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
-    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles),
-               _ptr(num_tiles), _stream()), "moe_route")
+    _need(1 <= keep <= groups <= 64 and experts % groups == 0 and (keep == groups or keep * (experts // groups) >= top),
+          f"moe_route: {keep} of {groups} groups of {experts} experts for top {top}")
+    fn = _fn("moe", "vk_moe_route_grouped", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
+    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), 1 if all_scores else 0, _ptr(ids),
+               _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles), _ptr(num_tiles), _stream()), "moe_route")
 
 
 def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
                 order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, weights: torch.Tensor, top: int,
                 limit: float, alpha: float, act: torch.Tensor, pair_out: torch.Tensor, residual: torch.Tensor) -> None:
     """The chosen experts of every token: ``y = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(Wg h, limit)`` and
-    ``u = clamp(Wu h, -limit, limit)``, then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])``."""
+    ``u = clamp(Wu h, -limit, limit)``, or with an infinite ``limit`` ``y = g * sigmoid(alpha * g) * u`` (alpha 1:
+    ``silu(g) * u``); then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])``."""
     _dev(h, w_gate, w_up, w_down, offsets, order, tiles, num_tiles, weights, act, pair_out, residual)
     tokens, width = h.shape
     experts, ff, _ = w_gate.shape
@@ -1184,3 +1194,217 @@ def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_dow
     _status(fn(_ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _dt(h, "h"), _ptr(offsets), _ptr(order),
                _ptr(tiles), _ptr(num_tiles), _ptr(weights), tokens, experts, top, width, ff, float(limit), float(alpha),
                _ptr(act), _ptr(pair_out), _ptr(residual), _stream()), "moe_experts")
+
+
+# --- norms behind a sublayer, sums of two streams, activations ------------------------------------------
+def _f32s(tensor: torch.Tensor, what: str) -> None:
+    """32-bit with unit inner stride; rows may lie further apart than they are long (a view of some columns)."""
+    _need(tensor.dtype == torch.float32 and tensor.stride(-1) == 1, f"{what} must be float32 with a unit inner stride")
+
+
+def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor) -> None:
+    """``residual += y / sqrt(mean(y^2) + eps) * weight`` row by row, all 32-bit."""
+    _dev(y, weight, residual)
+    _f32(y, "rmsnorm_add: y")
+    _f32(residual, "rmsnorm_add: residual")
+    rows, width = residual.shape
+    _need(y.shape == residual.shape and y.is_contiguous() and residual.is_contiguous(), "rmsnorm_add: shapes")
+    _need(weight.dtype == torch.float32 and weight.numel() == width and weight.is_contiguous(), "rmsnorm_add: weight")
+    fn = _fn("elementwise", "vk_rmsnorm_add", [_p, _p, _p, _i, _i, _f, _p])
+    _status(fn(_ptr(y), _ptr(weight), _ptr(residual), rows, width, float(eps), _stream()), "rmsnorm_add")
+
+
+def axpby(x: torch.Tensor, a: float, y: torch.Tensor, b: float, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``out (+)= a * x + b * y``, elementwise, 32-bit."""
+    _dev(x, y, out)
+    for t, what in ((x, "x"), (y, "y"), (out, "out")):
+        _f32(t, "axpby: " + what)
+        _need(t.is_contiguous() and t.numel() == out.numel(), "axpby: three contiguous tensors of one size")
+    fn = _fn("elementwise", "vk_axpby", [_p, _f, _p, _f, _p, _ll, _i, _p])
+    _status(fn(_ptr(x), float(a), _ptr(y), float(b), _ptr(out), out.numel(), 1 if accumulate else 0, _stream()), "axpby")
+
+
+ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "sigmoid": 4}
+
+
+def activation(x: torch.Tensor, kind: str, out: torch.Tensor, mul: Optional[torch.Tensor] = None) -> None:
+    """``out = act(x) (* mul)`` elementwise; ``x`` and ``mul`` may be row-strided views of either dtype, ``out`` is
+    contiguous.  ``kind``: none (a change of type), relu2 (the square of relu), silu, gelu_tanh, sigmoid."""
+    _dev(x, out, mul)
+    _need(kind in ACTIVATIONS, f"activation: kind {kind!r}; known: {', '.join(ACTIVATIONS)}")
+    rows, width = out.shape
+    _need(x.shape == out.shape and x.stride(1) == 1 and out.is_contiguous(), "activation: shapes")
+    if mul is not None:
+        _need(mul.shape == out.shape and mul.stride(1) == 1, "activation: the factor's shape")
+    fn = _fn("elementwise", "vk_activation", [_p, _i, _ll, _p, _i, _ll, _p, _i, _i, _i, _i, _p])
+    _status(fn(_ptr(x), _dt(x, "x"), x.stride(0), _ptr(mul), _dt(mul, "mul") if mul is not None else 0,
+               mul.stride(0) if mul is not None else 0, _ptr(out), _dt(out, "out"), rows, width, ACTIVATIONS[kind],
+               _stream()), "activation")
+
+
+def whole_norm_pack(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                    heads: int, kv_heads: int, dim: int, vdim: int, padded: int, qkv: torch.Tensor) -> None:
+    """From the 32-bit sums ``proj [T, >= q | k | v]``: q and k each divided by the root mean square of the whole
+    projection (all heads at once) and multiplied by their weights (None: left as they are), and q, k and v laid out
+    head by head, each padded with zeros to ``padded`` columns, as ``qkv [T, (heads + 2 kv_heads) * padded]``."""
+    _dev(proj, q_weight, k_weight, qkv)
+    _f32s(proj, "whole_norm_pack: proj")
+    tokens = qkv.shape[0]
+    need = (heads + kv_heads) * dim + kv_heads * vdim
+    _need(proj.dim() == 2 and proj.shape[0] == tokens and proj.shape[1] >= need and proj.stride(1) == 1,
+          "whole_norm_pack: proj")
+    _need(padded >= max(dim, vdim) and qkv.shape == (tokens, (heads + 2 * kv_heads) * padded) and qkv.is_contiguous(),
+          "whole_norm_pack: qkv")
+    for weight, count in ((q_weight, heads * dim), (k_weight, kv_heads * dim)):
+        if weight is not None:
+            _need(weight.dtype == torch.float32 and weight.numel() == count and weight.is_contiguous(),
+                  "whole_norm_pack: a weight per number of the projection")
+    fn = _fn("elementwise", "vk_whole_norm_pack", [_p, _ll, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, dim, vdim,
+               padded, _ptr(qkv), _dt(qkv, "qkv"), _stream()), "whole_norm_pack")
+
+
+def head_unpack_gate(attn: torch.Tensor, gate: Optional[torch.Tensor], gate_kind: str, heads: int, vdim: int,
+                     padded: int, out: torch.Tensor) -> None:
+    """``out[t, h * vdim + d] = attn[t, h * padded + d] * act(gate[t, h * vdim + d])``: the attention's output taken
+    out of its padded heads and, with ``gate`` (32-bit, row-strided), gated."""
+    _dev(attn, gate, out)
+    tokens = out.shape[0]
+    _need(attn.shape == (tokens, heads * padded) and attn.is_contiguous() and out.shape == (tokens, heads * vdim)
+          and out.is_contiguous() and out.dtype == attn.dtype and padded >= vdim, "head_unpack_gate: shapes")
+    _need(gate_kind in ACTIVATIONS, "head_unpack_gate: the gate's activation")
+    if gate is not None:
+        _f32s(gate, "head_unpack_gate: gate")
+        _need(gate.shape == out.shape and gate.stride(1) == 1, "head_unpack_gate: gate")
+    fn = _fn("elementwise", "vk_head_unpack_gate", [_p, _i, _p, _ll, _i, _i, _i, _i, _i, _p, _p])
+    _status(fn(_ptr(attn), _dt(attn, "attn"), _ptr(gate), gate.stride(0) if gate is not None else 0,
+               ACTIVATIONS[gate_kind], tokens, heads, vdim, padded, _ptr(out), _stream()), "head_unpack_gate")
+
+
+# --- recurrences with a diagonal decay ------------------------------------------------------------------
+DECAY_RULE_MAX_KEY_DIM = 256
+SELECTIVE_SCAN_MAX_STATES = 256
+
+
+def _lanes_share(n: int) -> int:
+    return 1 if n <= 16 else 2 if n <= 32 else 4 if n <= 64 else 8 if n <= 128 else 16
+
+
+def decay_rule_head_floats(dim: int, vdim: int) -> int:
+    """Floats of one head's state as :func:`decay_rule` keeps it (the key channels padded)."""
+    return vdim * 16 * _lanes_share(dim)
+
+
+def selective_scan_channel_floats(states: int) -> int:
+    """Floats of one channel's state as :func:`selective_scan` keeps it (padded)."""
+    return 16 * _lanes_share(states)
+
+
+def decay_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, silu_inputs: bool, decay: torch.Tensor,
+               state: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor, slots: torch.Tensor,
+               heads: int, dim: int, vdim: int, out: torch.Tensor, num_entries: int) -> None:
+    """Linear attention with a fixed decay per head, ``S <- decay S + k v^T; o = S^T q``, over the step's entries in
+    32-bit; ``q`` and ``k`` are row-strided views ``[T, heads * dim]`` with one stride, ``v [T, heads * vdim]``;
+    ``silu_inputs``: all three pass through silu as they are read.  ``state [slots + 1, floats]`` starts with
+    ``heads * decay_rule_head_floats(dim, vdim)`` floats of this layer."""
+    _dev(q, k, v, decay, state, entry_start, entry_first_pos, slots, out)
+    tokens = out.shape[0]
+    for t, what in ((q, "q"), (k, "k"), (v, "v"), (decay, "decay"), (state, "state"), (out, "out")):
+        _f32s(t, "decay_rule: " + what)
+    _need(q.shape == (tokens, heads * dim) and k.shape == q.shape and q.stride(1) == 1 and k.stride(1) == 1
+          and q.stride(0) == k.stride(0), "decay_rule: q and k")
+    _need(v.shape == (tokens, heads * vdim) and v.stride(1) == 1 and out.shape == v.shape and out.is_contiguous(),
+          "decay_rule: v and out")
+    _need(decay.numel() == heads and decay.is_contiguous(), "decay_rule: a decay per head")
+    _need(state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= heads * decay_rule_head_floats(dim, vdim),
+          "decay_rule: state row too short")
+    if dim > DECAY_RULE_MAX_KEY_DIM:
+        raise UnsupportedError(f"decay_rule: a key width of {dim} is above the kernel's limit of {DECAY_RULE_MAX_KEY_DIM}")
+    _i32(entry_start, entry_first_pos, slots)
+    _entries_ok((entry_start, entry_first_pos, slots), num_entries)
+    fn = _fn("scan", "vk_decay_rule", [_p, _p, _ll, _p, _ll, _i, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _p])
+    _status(fn(_ptr(q), _ptr(k), q.stride(0), _ptr(v), v.stride(0), 1 if silu_inputs else 0, _ptr(decay), _ptr(state),
+               state.stride(0), _ptr(entry_start), _ptr(entry_first_pos), _ptr(slots), num_entries, heads, dim, vdim,
+               _ptr(out), _stream()), "decay_rule")
+
+
+def gated_norm(x: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_kind: str, eps: float,
+               out: torch.Tensor) -> None:
+    """``out = x / rms(x) * weight * act(gate)`` over whole rows; ``x`` 32-bit, ``gate`` a 32-bit row-strided view."""
+    _dev(x, weight, gate, out)
+    _f32(x, "gated_norm: x")
+    _f32s(gate, "gated_norm: gate")
+    tokens, width = x.shape
+    _need(x.is_contiguous() and out.shape == x.shape and out.is_contiguous() and gate.shape == x.shape
+          and gate.stride(1) == 1, "gated_norm: shapes")
+    _need(weight.dtype == torch.float32 and weight.numel() == width and weight.is_contiguous(), "gated_norm: weight")
+    kinds = {"none": 0, "silu": 1, "sigmoid": 2}
+    _need(gate_kind in kinds, "gated_norm: the gate's activation")
+    fn = _fn("scan", "vk_gated_norm", [_p, _p, _p, _ll, _i, _f, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(x), _ptr(weight), _ptr(gate), gate.stride(0), kinds[gate_kind], float(eps), tokens, width, _ptr(out),
+               _dt(out, "out"), _stream()), "gated_norm")
+
+
+def causal_conv(x: torch.Tensor, conv: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                conv_offset: int, entry_of: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
+                slots: torch.Tensor, out32: torch.Tensor, out_run: Optional[torch.Tensor], num_entries: int) -> None:
+    """``y[t, c] = silu(bias[c] + sum_j conv[c, j] x[t - (taps - 1 - j), c])`` per entry, with the inputs before the
+    entry's first token from the state row (``(taps - 1) * C`` floats from ``conv_offset`` on; zeros at position 0),
+    which afterwards holds the entry's last inputs.  ``x``: a 32-bit row-strided view ``[T, C]``; ``out32`` 32-bit
+    and, if given, ``out_run`` the same in another dtype."""
+    _dev(x, conv, bias, state, entry_of, entry_start, entry_first_pos, slots, out32, out_run)
+    tokens, channels = out32.shape
+    taps = conv.shape[1]
+    _f32s(x, "causal_conv: x")
+    _f32(conv, "causal_conv: conv")
+    _f32s(state, "causal_conv: state")
+    _f32(out32, "causal_conv: out32")
+    _need(x.shape == (tokens, channels) and x.stride(1) == 1 and out32.is_contiguous(), "causal_conv: shapes")
+    _need(conv.shape == (channels, taps) and conv.is_contiguous() and taps >= 1, "causal_conv: conv must be [C, taps]")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == channels and bias.is_contiguous(), "causal_conv: bias")
+    if out_run is not None:
+        _need(out_run.shape == out32.shape and out_run.is_contiguous(), "causal_conv: out_run")
+    _need(state.dim() == 2 and state.stride(1) == 1 and conv_offset >= 0
+          and state.shape[1] >= conv_offset + (taps - 1) * channels, "causal_conv: state row too short")
+    _i32(entry_of, entry_start, entry_first_pos, slots)
+    _need(entry_of.numel() >= tokens, "causal_conv: entry_of")
+    _entries_ok((entry_start, entry_first_pos, slots), num_entries)
+    fn = _fn("scan", "vk_causal_conv", [_p, _ll, _p, _p, _i, _i, _p, _ll, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _i, _p])
+    _status(fn(_ptr(x), x.stride(0), _ptr(conv), _ptr(bias), taps, channels, _ptr(state), state.stride(0), conv_offset,
+               _ptr(entry_of), _ptr(entry_start), _ptr(entry_first_pos), _ptr(slots), tokens, num_entries, _ptr(out32),
+               _ptr(out_run), _dt(out_run, "out_run") if out_run is not None else 0, _stream()), "causal_conv")
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, b: torch.Tensor, c: torch.Tensor,
+                   a_log: torch.Tensor, skip: torch.Tensor, z: torch.Tensor, state: torch.Tensor,
+                   entry_start: torch.Tensor, entry_first_pos: torch.Tensor, slots: torch.Tensor, out: torch.Tensor,
+                   num_entries: int) -> None:
+    """The selective scan over the step's entries in 32-bit: per channel ``c`` and state ``n``
+    ``step = softplus(dt + dt_bias); S <- exp(step * -exp(a_log)) S + step x b; y = S . c + skip x``, and
+    ``out = y * silu(z)``.  ``x [T, C]`` contiguous; ``dt``, ``z`` row-strided views ``[T, C]``; ``b`` and ``c``
+    row-strided views ``[T, N]`` of one buffer; ``state`` starts with ``C * selective_scan_channel_floats(N)`` floats."""
+    _dev(x, dt, dt_bias, b, c, a_log, skip, z, state, entry_start, entry_first_pos, slots, out)
+    tokens, channels = x.shape
+    states = a_log.shape[1]
+    for t, what in ((x, "x"), (dt, "dt"), (dt_bias, "dt_bias"), (b, "b"), (c, "c"), (a_log, "a_log"), (skip, "skip"),
+                    (z, "z"), (state, "state")):
+        _f32s(t, "selective_scan: " + what)
+    _need(x.is_contiguous() and dt.shape == x.shape and dt.stride(1) == 1 and z.shape == x.shape and z.stride(1) == 1
+          and out.shape == x.shape and out.is_contiguous(), "selective_scan: x, dt, z, out")
+    _need(b.shape == (tokens, states) and c.shape == b.shape and b.stride(1) == 1 and c.stride(1) == 1
+          and b.stride(0) == c.stride(0), "selective_scan: b and c")
+    _need(a_log.shape == (channels, states) and a_log.is_contiguous() and dt_bias.numel() == channels
+          and dt_bias.is_contiguous() and skip.numel() == channels and skip.is_contiguous(), "selective_scan: parameters")
+    if states > SELECTIVE_SCAN_MAX_STATES:
+        raise UnsupportedError(f"selective_scan: {states} states a channel are above the kernel's limit of "
+                               f"{SELECTIVE_SCAN_MAX_STATES}")
+    _need(state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= channels * selective_scan_channel_floats(states), "selective_scan: state row too short")
+    _i32(entry_start, entry_first_pos, slots)
+    _entries_ok((entry_start, entry_first_pos, slots), num_entries)
+    fn = _fn("scan", "vk_selective_scan", [_p, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _ll, _p, _ll, _p, _p, _p, _i, _i, _i,
+                                           _p, _i, _p])
+    _status(fn(_ptr(x), _ptr(dt), dt.stride(0), _ptr(dt_bias), _ptr(b), _ptr(c), b.stride(0), _ptr(a_log), _ptr(skip),
+               _ptr(z), z.stride(0), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first_pos), _ptr(slots),
+               num_entries, channels, states, _ptr(out), _dt(out, "out"), _stream()), "selective_scan")

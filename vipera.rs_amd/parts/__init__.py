@@ -1,4 +1,4 @@
-from . import attention, block, embedding, latent, mlp, moe, norm, recurrent, rotary  # noqa: F401  (registers the built-in kinds)
+from . import attention, block, embedding, latent, mlp, moe, norm, pair, recurrent, rotary  # noqa: F401  (registers the built-in kinds)
 from .base import (
     Block, FeedForward, KVCacheSpec, Mixer, Norm, NormHandoff, Part, PositionEncoding, StateSpec, part_class,
     register_block, register_embedding, register_ffn, register_head, register_mixer, register_norm,

@@ -5,6 +5,15 @@ Order of work as in the reference's batched pass (crates/vipera-backend-cpu/src/
 cache; attend causally by count (a token at position p reads positions ``<= p`` of its own request,
 or the last ``window`` of them); ``x += attn Wo^T``.  The three projections run as one product over
 the concatenated weight ``[Wq; Wk; Wv]``, whose rows equal the separate products' rows.
+
+Options, each a parameter that any architecture may set: ``softcap`` (a score becomes ``softcap * tanh(score /
+softcap)``); ``chunk`` (a token sees the earlier tokens of its own block of that many positions, blocks counted from
+position 0, instead of a window); ``value_dim`` (values narrower or wider than keys); ``qk_norm: "whole"`` (q and k
+each RMS-normed over the whole projection, all heads at once, with a weight per number, before the rotation);
+``gate: "sigmoid"`` (the heads' outputs times ``sigmoid(Wg h)`` before the output projection); ``tensors`` (the
+tensors' names after the part's name).  With any of the last three the step runs as one product ``[q | k | v | g]`` with
+32-bit sums, a kernel that norms and lays the heads out at one padded width, the rotation with the cache write, the
+paged attention kernels at that width, and a kernel that unpacks and gates.
 """
 from __future__ import annotations
 
@@ -29,6 +38,30 @@ def _cat(tensors: List[torch.Tensor]) -> torch.Tensor:
     return torch.cat(tensors, dim=0).contiguous()
 
 
+_DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                  "g": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+
+
+def _tensor_names(p) -> Dict[str, str]:
+    names = dict(_DEFAULT_NAMES)
+    names.update(p.get("tensors") or {})
+    return names
+
+
+def _is_general(p) -> bool:
+    """Whether the layer needs the path that norms, pads and gates (see the module's text)."""
+    return bool(p.get("qk_norm") or p.get("gate") or int(p.get("value_dim") or p["head_dim"]) != int(p["head_dim"]))
+
+
+def _padded_width(p) -> int:
+    """The one width that keys and values have in the cache and in the attention kernels: the head width, or with
+    values of another width the larger of the two, rounded up to a multiple of 16."""
+    head_dim = int(p["head_dim"])
+    if not _is_general(p):
+        return head_dim
+    return (max(head_dim, int(p.get("value_dim") or head_dim)) + 15) // 16 * 16
+
+
 class Attention(Mixer):
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
@@ -40,48 +73,78 @@ class Attention(Mixer):
         self.window = int(p.get("window") or 0)
         self.qkv_bias = bool(p.get("qkv_bias", False))
         self.out_bias = bool(p.get("out_bias", False))
+        self.softcap = float(p.get("softcap") or 0.0)
+        self.chunk = int(p.get("chunk") or 0)
+        if self.chunk and self.window:
+            raise InvalidArgumentError("attention: a window and blocks of positions exclude each other")
+        self.mask = -self.chunk if self.chunk else self.window      # what the kernels take as `window`
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.qk_norm, self.gate = p.get("qk_norm"), p.get("gate")
+        self.general = _is_general(p)
+        self.padded = _padded_width(p)
+        if self.general and (self.qkv_bias or self.out_bias):
+            raise UnsupportedError("attention: biases with value_dim, qk_norm or gate are not implemented")
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         if self.heads % self.kv_heads:
             raise InvalidArgumentError(f"heads {self.heads} is not a multiple of kv_heads {self.kv_heads}")
         self.q_width = self.heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
-        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = None
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
         p = spec.params
         base = f"{prefix}{p['name']}."
+        names = _tensor_names(p)
         hidden, hd = int(p["hidden"]), int(p["head_dim"])
+        vd = int(p.get("value_dim") or hd)
         q, kv = int(p["heads"]) * hd, int(p["kv_heads"]) * hd
         specs: List[TensorSpec] = []
-        for name, rows in (("q", q), ("k", kv), ("v", kv)):
-            specs.append(TensorSpec(f"{base}{name}_proj.weight", (rows, hidden), MATRIX))
+        for name, rows in (("q", q), ("k", kv), ("v", int(p["kv_heads"]) * vd)):
+            specs.append(TensorSpec(base + names[name], (rows, hidden), MATRIX))
             if p.get("qkv_bias"):
                 specs.append(TensorSpec(f"{base}{name}_proj.bias", (rows,), VECTOR))
-        specs.append(TensorSpec(base + "o_proj.weight", (hidden, q), MATRIX))
+        specs.append(TensorSpec(base + names["o"], (hidden, int(p["heads"]) * vd), MATRIX))
         if p.get("out_bias"):
             specs.append(TensorSpec(base + "o_proj.bias", (hidden,), VECTOR))
+        if p.get("qk_norm"):
+            specs += [TensorSpec(base + names["q_norm"], (q,), VECTOR, "one_plus_normal"),
+                      TensorSpec(base + names["k_norm"], (kv,), VECTOR, "one_plus_normal")]
+        if p.get("gate"):
+            specs.append(TensorSpec(base + names["g"], (int(p["heads"]) * vd, hidden), MATRIX))
         return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
-        self.w_qkv = _cat([tensors[base + f"{n}_proj.weight"] for n in "qkv"])
+        names = _tensor_names(self.spec.params)
+        parts = [tensors[base + names[n]] for n in "qkv"]
+        if self.gate:
+            parts.append(tensors[base + names["g"]])
+        self.w_qkv = _cat(parts)
         if self.qkv_bias:
             self.b_qkv = torch.cat([tensors[base + f"{n}_proj.bias"] for n in "qkv"]).contiguous()
-        self.w_o = tensors[base + "o_proj.weight"]
+        self.w_o = tensors[base + names["o"]]
         if self.out_bias:
             self.b_o = tensors[base + "o_proj.bias"]
+        if self.qk_norm:
+            self.q_norm, self.k_norm = tensors[base + names["q_norm"]], tensors[base + names["k_norm"]]
 
     @classmethod
     def declare_cache(cls, spec: PartSpec):
         p = spec.params
-        return KVCacheSpec(int(p["kv_heads"]), int(p["head_dim"]), int(p.get("window") or 0)), None
+        # blocks of positions keep everything: a page is only ever passed by all tokens at a block's edge, and the
+        # pool is sized for whole requests
+        return KVCacheSpec(int(p["kv_heads"]), _padded_width(p), int(p.get("window") or 0)), None
 
     @classmethod
     def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
         p = spec.params
-        heads, kv_heads, head_dim = int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        heads, kv_heads, head_dim = int(p["heads"]), int(p["kv_heads"]), _padded_width(p)
+        if p.get("qk_norm") not in (None, "whole"):
+            raise UnsupportedError(f"attention: qk_norm {p.get('qk_norm')!r} is not implemented; \"whole\" or none")
+        if p.get("gate") not in (None, "sigmoid", "silu"):
+            raise UnsupportedError(f"attention: gate {p.get('gate')!r} is not implemented; \"sigmoid\", \"silu\" or none")
         if head_dim > kernels.ATTENTION_MAX_HEAD_DIM:
             raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of "
                                    f"{kernels.ATTENTION_MAX_HEAD_DIM}")
@@ -90,6 +153,7 @@ class Attention(Mixer):
                                    f"kernels' limit of {kernels.ATTENTION_MAX_HEADS} heads in all")
 
     fills_handoff = True
+    can_overwrite = True
 
     def _fused(self, tokens: int, position, batch) -> Optional[str]:
         """How product, rotation and cache write of a step of ``tokens`` run as one launch sequence without a
@@ -98,6 +162,8 @@ class Attention(Mixer):
         kernel (no table of the step's angles)."""
         fused = position.fused_rotary()
         n, k = self.w_qkv.shape
+        if self.general:
+            return None
         if not (fused is not None and fused[1] == self.head_dim and self.runtime.dtype == torch.bfloat16
                 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 2 == 0 and k % 8 == 0
                 and position.step_angles(batch) is None):
@@ -112,9 +178,41 @@ class Attention(Mixer):
         # the fused products can divide by the norm themselves
         return self._fused(tokens, position, batch) is not None
 
-    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None,
-                incoming=None) -> None:
+    def _forward_general(self, h, batch, cache, position, residual, reads_only: bool, accumulate: bool) -> None:
+        """q and k normed over the whole projection, values of another width, a gate on the output: see the module's
+        text.  Heads are ``padded`` wide in the buffers that the rotation and the attention kernels see."""
         tokens = residual.shape[0]
+        width = self.padded
+        proj = torch.empty((tokens, self.w_qkv.shape[0]), dtype=torch.float32, device=residual.device)
+        linear(h, self.w_qkv, None, proj)
+        qkv = self.runtime.empty((tokens, (self.heads + 2 * self.kv_heads) * width))
+        kernels.whole_norm_pack(proj, self.q_norm, self.k_norm, float(self.spec.params.get("eps") or 0.0), self.heads,
+                                self.kv_heads, self.head_dim, self.value_dim, width, qkv)
+        table = batch.block_tables[cache.group]
+        fused = position.fused_rotary()
+        inv_freq, rotary_dim = fused if fused is not None else (None, 0)
+        if fused is None:
+            position.apply(qkv, batch, self.heads, self.kv_heads, width)
+        angles = position.step_angles(batch) if rotary_dim else None
+        if not reads_only:
+            kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
+                                 table, self.heads, self.kv_heads, width, angles)
+        elif rotary_dim:
+            kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, None, None, batch.entry_of_token, None,
+                                 self.heads, self.kv_heads, width, angles)
+        attn = self.runtime.empty((tokens, self.heads * width))
+        paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, width, self.scale,
+                        self.mask, self.softcap)
+        values = self.runtime.empty((tokens, self.heads * self.value_dim))
+        gate = proj[:, (self.heads + self.kv_heads) * self.head_dim + self.kv_heads * self.value_dim:] if self.gate else None
+        kernels.head_unpack_gate(attn, gate, self.gate or "none", self.heads, self.value_dim, width, values)
+        linear(values, self.w_o, None, residual, accumulate=accumulate)
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None,
+                incoming=None, accumulate: bool = True) -> None:
+        tokens = residual.shape[0]
+        if self.general:
+            return self._forward_general(h, batch, cache, position, residual, reads_only, accumulate)
         how = self._fused(tokens, position, batch)
         if incoming is not None and how is None:
             raise UnsupportedError("attention was handed a split norm for a step whose product cannot divide by it")
@@ -148,13 +246,13 @@ class Attention(Mixer):
                                      None, self.heads, self.kv_heads, self.head_dim, angles)
         attn = self.runtime.empty((tokens, self.q_width))
         paged_attention(qkv, cache.k, cache.v, attn, batch, table, self.heads, self.kv_heads, self.head_dim,
-                        self.scale, self.window)
+                        self.scale, self.mask, self.softcap)
         if handoff is not None:
             # the output product also prepares the norm that follows (its gained copy of the residual, its squares)
             # where its kernel can; 0 groups say that it could not
             handoff.groups = linear_follow(attn, self.w_o, self.b_o, residual, handoff.gain, handoff.scaled, handoff.sumsq)
         else:
-            linear(attn, self.w_o, self.b_o, residual, accumulate=True)
+            linear(attn, self.w_o, self.b_o, residual, accumulate=accumulate)
 
 
 register_mixer("attention", Attention)

@@ -120,6 +120,10 @@ class Norm(Part):
         """A :class:`NormHandoff` for ``tokens`` rows if this norm can be split between its neighbours, else None."""
         return None
 
+    def add_into(self, y: torch.Tensor, residual: torch.Tensor) -> None:
+        """``residual += norm(y)`` in 32-bit: what a block calls for a norm that stands behind a sublayer."""
+        raise NotImplementedError
+
 
 class PositionEncoding(Part):
     def fused_rotary(self):
@@ -155,11 +159,18 @@ class Mixer(Part):
         None) for a step of ``tokens`` rows."""
         return False
 
+    #: a mixer that sets this takes ``accumulate=False`` in ``forward`` and then writes its output into ``residual``
+    #: instead of adding to it (a block with a norm behind the mixer hands it a buffer that need not be cleared)
+    can_overwrite = False
+
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    #: as :attr:`Mixer.can_overwrite`
+    can_overwrite = False
+
     #: a feed-forward that sets this takes ``outgoing=`` in ``forward`` and may fill it for the next layer's first norm
     fills_handoff = False
 

@@ -3,6 +3,9 @@
 ``prenorm``: ``x += mixer(norm_1(x)); x += ffn(norm_2(x))``, the pre-norm residual block of the
 reference (crates/vipera-backend-cpu/src/model.rs:3-4, 975-1198).
 ``parallel``: ``h = norm(x); x += mixer(h) + ffn(h)``.
+``sandwich``: a norm before and behind each sublayer, ``x += norm_1b(mixer(norm_1(x))); x += norm_2b(ffn(norm_2(x)))``,
+and optionally a part that adds to the stream after both (``extras["after"]``, of the feed-forward family; it reads the
+32-bit stream itself).  The norms behind the sublayers are ``extras["mixer_post_norm"]`` and ``extras["ffn_post_norm"]``.
 """
 from __future__ import annotations
 
@@ -110,5 +113,68 @@ class ParallelBlock(Block):
         self.ffn.forward(h, batch, x)
 
 
+class SandwichBlock(Block):
+    """See the module's text.  A sublayer's output goes into a 32-bit buffer of its own (written, where the part can,
+    instead of cleared and added to), is normed there and added to the stream by one kernel."""
+
+    def __init__(self, spec: LayerSpec, runtime):
+        super().__init__(spec, runtime)
+        self.parts = {}
+        for role, family, part in self._roles(spec):
+            self.parts[role] = part_class(family, part.kind)(part, spec.prefix, runtime)
+        self.mixer = self.parts["mixer"]
+        self.has_ffn = spec.ffn.kind != "none"
+
+    @classmethod
+    def _roles(cls, spec: LayerSpec):
+        roles = [("mixer_norm", "norm", spec.mixer_norm), ("mixer", "mixer", spec.mixer),
+                 ("mixer_post_norm", "norm", spec.extras["mixer_post_norm"]), ("position", "position", spec.position)]
+        if spec.ffn.kind != "none":
+            roles += [("ffn_norm", "norm", spec.ffn_norm), ("ffn", "ffn", spec.ffn),
+                      ("ffn_post_norm", "norm", spec.extras["ffn_post_norm"])]
+        if "after" in spec.extras:
+            roles.append(("after", "ffn", spec.extras["after"]))
+        return roles
+
+    @classmethod
+    def declare(cls, spec: LayerSpec) -> List[TensorSpec]:
+        out: List[TensorSpec] = []
+        for _, family, part in cls._roles(spec):
+            out += part_class(family, part.kind).declare(part, spec.prefix)
+        return out
+
+    @classmethod
+    def check_supported(cls, spec: LayerSpec, dtype) -> None:
+        for _, family, part in cls._roles(spec):
+            part_class(family, part.kind).check_supported(part, dtype)
+
+    def load(self, tensors) -> None:
+        for part in self.parts.values():
+            part.load(tensors)
+
+    def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
+        import torch
+        parts = self.parts
+        h = parts["mixer_norm"].forward(x)
+        if parts["mixer"].can_overwrite:
+            y = torch.empty_like(x)
+            parts["mixer"].forward(h, batch, cache, state, parts["position"], y, reads_only, accumulate=False)
+        else:
+            y = torch.zeros_like(x)
+            parts["mixer"].forward(h, batch, cache, state, parts["position"], y, reads_only)
+        parts["mixer_post_norm"].add_into(y, x)
+        if self.has_ffn:
+            h = parts["ffn_norm"].forward(x)
+            if parts["ffn"].can_overwrite:
+                parts["ffn"].forward(h, batch, y, accumulate=False)
+            else:
+                y.zero_()
+                parts["ffn"].forward(h, batch, y)
+            parts["ffn_post_norm"].add_into(y, x)
+        if "after" in parts:
+            parts["after"].forward(None, batch, x)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("sandwich", SandwichBlock)
 register_block("parallel", ParallelBlock)

@@ -87,5 +87,51 @@ class NoFeedForward(FeedForward):
         return None
 
 
+class PlainMLP(FeedForward):
+    """``x += Wdown act(Wup h)`` without a gate.  ``params``: ``hidden``, ``intermediate``, ``activation`` ("relu2":
+    the square of relu; "silu"; "gelu_tanh"), ``name``; tensors ``<name>.up`` and ``<name>.down`` (or as
+    ``params["tensors"]`` names them)."""
+
+    can_overwrite = True
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        self.hidden, self.inter = int(spec.params["hidden"]), int(spec.params["intermediate"])
+        self.activation = spec.params.get("activation", "relu2")
+        self.w_up = self.w_down = None
+
+    @staticmethod
+    def _names(spec: PartSpec, prefix: str):
+        names = {"up": "up", "down": "down"}
+        names.update(spec.params.get("tensors") or {})
+        base = f"{prefix}{spec.params['name']}."
+        return base + names["up"], base + names["down"]
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        up, down = cls._names(spec, prefix)
+        hidden, inter = int(spec.params["hidden"]), int(spec.params["intermediate"])
+        return [TensorSpec(up, (inter, hidden), MATRIX), TensorSpec(down, (hidden, inter), MATRIX)]
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype) -> None:
+        kind = spec.params.get("activation", "relu2")
+        if kind not in ("relu2", "silu", "gelu_tanh"):
+            raise UnsupportedError(f"mlp: activation {kind!r} is not implemented; relu2, silu or gelu_tanh")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        up, down = self._names(self.spec, self.prefix)
+        self.w_up, self.w_down = tensors[up], tensors[down]
+
+    def forward(self, h, batch, residual, accumulate: bool = True, **_unused) -> None:
+        tokens = residual.shape[0]
+        up = self.runtime.empty((tokens, self.inter))
+        linear(h, self.w_up, None, up)
+        act = self.runtime.empty((tokens, self.inter))
+        kernels.activation(up, self.activation, act)
+        linear(act, self.w_down, None, residual, accumulate=accumulate)
+
+
+register_ffn("mlp", PlainMLP)
 register_ffn("gated_mlp", GatedMLP)
 register_ffn("none", NoFeedForward)

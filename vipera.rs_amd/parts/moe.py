@@ -3,7 +3,11 @@
 Router logits ``z = W_router h`` in 32-bit; the ``top`` largest are chosen (the lowest id among equals) and weighted
 by the softmax over the chosen logits only.  An expert computes ``g = min(W_gate h, limit)``,
 ``u = clamp(W_up h, -limit, limit)``, ``y = g * sigmoid(alpha * g) * (u + 1)`` and returns ``W_down y``; the layer
-adds the weighted sum of the chosen experts' outputs to the residual.  ``limit`` and ``alpha`` are parameters.
+adds the weighted sum of the chosen experts' outputs to the residual.  ``limit`` and ``alpha`` are parameters; without
+a ``limit`` nothing is clamped and ``y = g * sigmoid(alpha * g) * u`` (``alpha`` 1: ``silu(g) * u``).  ``groups`` and
+``keep``: the experts form that many equal groups of neighbours, a group's score is its largest logit, and only experts
+of the ``keep`` best groups can be chosen.  ``scores: "all"``: the weights are the chosen experts' shares of the softmax
+over all experts, not renormalized.
 
 The step's (token, choice) pairs are grouped by expert on the device, so nothing about the routing reaches the
 host and a step of single tokens can be captured; see ``csrc/kernels/moe.hip``.
@@ -23,16 +27,19 @@ from .base import FeedForward, register_ffn
 
 
 class MixtureOfExperts(FeedForward):
-    """``params``: ``hidden``, ``intermediate`` (an expert's width), ``experts``, ``top``, ``limit``, ``alpha``
-    (1.702 unless given), ``name``; tensors ``<name>.router`` and ``<name>.e<i>.gate | up | down``."""
+    """``params``: ``hidden``, ``intermediate`` (an expert's width), ``experts``, ``top``, ``limit`` (None: no clamp),
+    ``alpha`` (1.702 unless given), ``groups`` and ``keep`` (1 and 1 unless given), ``scores`` ("chosen" or "all"),
+    ``name``; tensors ``<name>.router`` and ``<name>.e<i>.gate | up | down``."""
 
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
         p = spec.params
         self.hidden, self.inter = int(p["hidden"]), int(p["intermediate"])
         self.experts, self.top = int(p["experts"]), int(p["top"])
-        self.limit = float(p["limit"])
+        self.limit = float(p["limit"]) if p.get("limit") is not None else float("inf")
         self.alpha = float(p.get("alpha", 1.702))
+        self.groups, self.keep = int(p.get("groups") or 1), int(p.get("keep") or p.get("groups") or 1)
+        self.all_scores = p.get("scores", "chosen") == "all"
         if not 1 <= self.top <= self.experts:
             raise InvalidArgumentError(f"a token cannot use {self.top} of {self.experts} experts")
         self.w_router = self.w_gate = self.w_up = self.w_down = None
@@ -56,6 +63,15 @@ class MixtureOfExperts(FeedForward):
         if top > 64 or experts > 4096:
             raise UnsupportedError(f"mixture of experts: top {top} of {experts} experts is above the routing kernel's "
                                    "limits of 64 of 4,096")
+        groups = int(spec.params.get("groups") or 1)
+        keep = int(spec.params.get("keep") or groups)
+        if groups > 64:
+            raise UnsupportedError(f"mixture of experts: {groups} groups are above the routing kernel's limit of 64")
+        if groups < 1 or experts % groups or not 1 <= keep <= groups or (keep < groups and keep * (experts // groups) < top):
+            raise InvalidArgumentError(f"mixture of experts: {keep} of {groups} groups of {experts} experts cannot "
+                                       f"give a token its {top}")
+        if spec.params.get("scores", "chosen") not in ("chosen", "all"):
+            raise UnsupportedError(f"mixture of experts: scores {spec.params.get('scores')!r}; \"chosen\" or \"all\"")
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
@@ -78,7 +94,8 @@ class MixtureOfExperts(FeedForward):
         num_tiles = ints[2 * pairs + self.experts + 1:2 * pairs + self.experts + 2]
         tiles = ints[2 * pairs + self.experts + 2:]
         weights = torch.empty(pairs, dtype=torch.float32, device=device)
-        kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles, tile_rows)
+        kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles, tile_rows,
+                          groups=self.groups, keep=self.keep, all_scores=self.all_scores)
         act = self.runtime.empty((pairs, self.inter))
         pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
         kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,

@@ -1,4 +1,6 @@
 """Norms.  RMSNorm: ``out = (x * rsqrt(mean(x^2) + eps)) * weight`` with the sum in 32-bit; Dynamic Tanh below.
+With ``one_plus`` the stored weight lies around zero and the gain is ``1 + weight`` (added once, in 32-bit, when the
+weight is loaded).  ``add_into`` is the norm behind a sublayer: the normed rows are added to the 32-bit residual.
 
 Reference: crates/vipera-backend-cpu/src/model.rs:4282-4288 (eps inside the square root, added to
 the mean; multiply order ``(x * inv) * w``).
@@ -16,19 +18,35 @@ from .base import Norm, NormHandoff, register_norm
 
 
 class RMSNorm(Norm):
+    """``params``: ``width``, ``eps``, ``name`` (the tensor is ``<name>.weight``, or ``params["tensor"]`` outright),
+    ``one_plus`` (the gain is 1 + the stored weight)."""
+
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
         self.width = int(spec.params["width"])
         self.eps = float(spec.params["eps"])
+        self.one_plus = bool(spec.params.get("one_plus"))
         self.weight: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def _tensor(spec: PartSpec, prefix: str) -> str:
+        return f"{prefix}{spec.params['tensor']}" if spec.params.get("tensor") else f"{prefix}{spec.params['name']}.weight"
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(f"{prefix}{spec.params['name']}.weight", (int(spec.params["width"]),), VECTOR,
-                           "one_plus_normal")]
+        return [TensorSpec(cls._tensor(spec, prefix), (int(spec.params["width"]),), VECTOR,
+                           "normal" if spec.params.get("one_plus") else "one_plus_normal",
+                           optional=bool(spec.params.get("optional")))]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[f"{self.prefix}{self.spec.params['name']}.weight"]
+        weight = tensors.get(self._tensor(self.spec, self.prefix))
+        if weight is not None and self.one_plus:
+            weight = (weight.float() + 1.0).contiguous()
+        self.weight = weight
+
+    def add_into(self, y: torch.Tensor, residual: torch.Tensor) -> None:
+        """``residual += y / rms(y) * gain``, all in 32-bit (the norm behind a sublayer)."""
+        kernels.rmsnorm_add(y, self.weight, self.eps, residual)
 
     def handoff(self, tokens: int) -> Optional[NormHandoff]:
         if self.runtime.dtype != torch.bfloat16 or self.weight is None or self.weight.dtype != torch.float32:

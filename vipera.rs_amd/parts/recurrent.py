@@ -10,7 +10,17 @@ dt_bias))`` per head; then per head ``S <- g S; u = beta (v - S^T k); S <- S + k
 ``w = exp(-exp(W2 tanh(W1 mix_w) + w0))`` per key channel; per head ``o = (S + diag(u) k v^T)^T r`` and then
 ``S <- diag(w) S + k v^T``; the read-out is ``o / rms(o) * norm * silu(Wg mix_g)`` and goes through ``Wo``.
 
-Both keep their state in 32-bit in the request's slot: the matrices, and what the next token needs of this one (the
+``decay_attention``: linear attention whose heads forget at a fixed rate each.  ``q = act(Wq h)``, ``k = act(Wk h)``
+(``heads x dim``), ``v = act(Wv h)`` (``heads x vdim``); per head ``S <- decay_h S + k v^T; o = S^T q``; the heads'
+outputs are normed together (one RMS norm over ``heads * vdim`` numbers), gated by ``sigmoid(Wg h)`` and go through
+``Wo``.
+
+``selective_scan``: Mamba.  ``W_in h = [x | z]``; x passes a short causal convolution per channel with a bias, and
+silu; ``W_x x = [dt | B | C]``; ``step = softplus(W_dt dt + dt_bias)``; per channel c and state n
+``S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c x_c B_n`` with ``A = -exp(A_log)``; ``y_c = S[c, :] . C + D_c x_c``;
+``y * silu(z)`` goes through ``Wo``.
+
+All keep their state in 32-bit in the request's slot: the matrices, and what the next token needs of this one (the
 convolution's last inputs; the last ``h``).  An entry that starts at position 0 starts from zeros.  Everything the
 kernels look at lies on the device, so a step of single tokens can be captured.
 """
@@ -202,5 +212,140 @@ class Wkv(Mixer):
         linear(gated, self.w_o, None, residual, accumulate=True)
 
 
+class DecayAttention(Mixer):
+    """``params``: ``hidden``, ``heads``, ``dim``, ``vdim``, ``decay`` (one number per head), ``eps`` (of the read-out's
+    norm), ``activation`` ("silu" or "none", of q, k and v), ``gate`` ("sigmoid", "silu" or "none"), ``name``; tensors
+    ``<name>.q | k | v | g | o | norm``."""
+
+    can_overwrite = True
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.heads, self.dim, self.vdim = int(p["hidden"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.eps = float(p["eps"])
+        self.activation, self.gate = p.get("activation", "silu"), p.get("gate", "sigmoid")
+        rates = [float(r) for r in p["decay"]]
+        if len(rates) != self.heads:
+            raise InvalidArgumentError(f"decay_attention: {len(rates)} decays for {self.heads} heads")
+        if self.activation not in ("silu", "none") or self.gate not in ("sigmoid", "silu", "none"):
+            raise UnsupportedError(f"decay_attention: activation {self.activation!r} with gate {self.gate!r} is not implemented")
+        self.decay = torch.tensor(rates, dtype=torch.float32, device=runtime.device)
+        self.qk, self.vw = self.heads * self.dim, self.heads * self.vdim
+        self.w_in = self.w_o = self.norm = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, qk, vw = int(p["hidden"]), int(p["heads"]) * int(p["dim"]), int(p["heads"]) * int(p["vdim"])
+        return [TensorSpec(base + "q", (qk, hidden), MATRIX), TensorSpec(base + "k", (qk, hidden), MATRIX),
+                TensorSpec(base + "v", (vw, hidden), MATRIX), TensorSpec(base + "g", (vw, hidden), MATRIX),
+                TensorSpec(base + "o", (hidden, vw), MATRIX),
+                TensorSpec(base + "norm", (vw,), VECTOR, "one_plus_normal")]
+
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        p = spec.params
+        return None, StateSpec((int(p["heads"]) * kernels.decay_rule_head_floats(int(p["dim"]), int(p["vdim"])),), torch.float32)
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        if int(spec.params["dim"]) > kernels.DECAY_RULE_MAX_KEY_DIM:
+            raise UnsupportedError(f"decay_attention: a key width of {spec.params['dim']} is above the kernel's limit of "
+                                   f"{kernels.DECAY_RULE_MAX_KEY_DIM}")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", "g")])     # one product for all that reads h
+        self.w_o, self.norm = tensors[base + "o"], tensors[base + "norm"]
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
+        tokens, entries = residual.shape[0], batch.num_entries
+        f32 = dict(dtype=torch.float32, device=residual.device)
+        proj = torch.empty((tokens, self.w_in.shape[0]), **f32)        # 32-bit from the product's sums on
+        linear(h, self.w_in, None, proj)
+        q, k = proj[:, :self.qk], proj[:, self.qk:2 * self.qk]
+        v, g = proj[:, 2 * self.qk:2 * self.qk + self.vw], proj[:, 2 * self.qk + self.vw:]
+        o = torch.empty((tokens, self.vw), **f32)
+        kernels.decay_rule(q, k, v, self.activation == "silu", self.decay, state, batch.entry_start,
+                           batch.entry_first_pos, batch.slots, self.heads, self.dim, self.vdim, o, entries)
+        gated = self.runtime.empty((tokens, self.vw))
+        kernels.gated_norm(o, self.norm, g, self.gate, self.eps, gated)
+        linear(gated, self.w_o, None, residual, accumulate=accumulate)
+
+
+class SelectiveScan(Mixer):
+    """``params``: ``hidden``, ``inner`` (channels), ``state`` (numbers per channel), ``dt_rank``, ``conv`` (taps),
+    ``name``; tensors ``<name>.in | conv | conv.b | x | dt | dt.b | A_log | D | o``."""
+
+    can_overwrite = True
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.inner, self.states = int(p["hidden"]), int(p["inner"]), int(p["state"])
+        self.rank, self.taps = int(p["dt_rank"]), int(p["conv"])
+        self.w_in = self.conv = self.conv_b = self.w_x = self.w_dt = self.dt_b = self.a_log = self.skip = self.w_o = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, inner, states, rank, taps = (int(p[k]) for k in ("hidden", "inner", "state", "dt_rank", "conv"))
+        return [TensorSpec(base + "in", (2 * inner, hidden), MATRIX),
+                TensorSpec(base + "conv", (inner, taps), VECTOR, std=0.5), TensorSpec(base + "conv.b", (inner,), VECTOR),
+                TensorSpec(base + "x", (rank + 2 * states, inner), MATRIX),
+                TensorSpec(base + "dt", (inner, rank), MATRIX, std=0.2), TensorSpec(base + "dt.b", (inner,), VECTOR, std=0.5),
+                TensorSpec(base + "A_log", (inner, states), VECTOR, std=0.5), TensorSpec(base + "D", (inner,), VECTOR, std=0.5),
+                TensorSpec(base + "o", (hidden, inner), MATRIX)]
+
+    @classmethod
+    def state_floats(cls, p) -> int:
+        return int(p["inner"]) * kernels.selective_scan_channel_floats(int(p["state"])) + (int(p["conv"]) - 1) * int(p["inner"])
+
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        return None, StateSpec((cls.state_floats(spec.params),), torch.float32)
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        p = spec.params
+        if int(p["state"]) > kernels.SELECTIVE_SCAN_MAX_STATES:
+            raise UnsupportedError(f"selective_scan: {p['state']} states a channel are above the kernel's limit of "
+                                   f"{kernels.SELECTIVE_SCAN_MAX_STATES}")
+        if int(p["conv"]) < 1 or int(p["dt_rank"]) < 1:
+            raise UnsupportedError("selective_scan: the convolution needs at least one tap and dt at least one row")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        self.w_in, self.w_x, self.w_dt, self.w_o = (tensors[base + n] for n in ("in", "x", "dt", "o"))
+        self.conv, self.conv_b, self.dt_b = tensors[base + "conv"], tensors[base + "conv.b"], tensors[base + "dt.b"]
+        self.a_log, self.skip = tensors[base + "A_log"], tensors[base + "D"]
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
+        tokens, entries = residual.shape[0], batch.num_entries
+        f32 = dict(dtype=torch.float32, device=residual.device)
+        xz = torch.empty((tokens, 2 * self.inner), **f32)
+        linear(h, self.w_in, None, xz)
+        matrices = self.inner * kernels.selective_scan_channel_floats(self.states)
+        # the convolved x enters the recurrence in 32-bit; the product behind it reads it in the run's dtype
+        x32 = torch.empty((tokens, self.inner), **f32)
+        x_run = None if self.runtime.dtype == torch.float32 else self.runtime.empty((tokens, self.inner))
+        kernels.causal_conv(xz[:, :self.inner], self.conv, self.conv_b, state, matrices, batch.entry_of_token,
+                            batch.entry_start, batch.entry_first_pos, batch.slots, x32, x_run, entries)
+        low = torch.empty((tokens, self.rank + 2 * self.states), **f32)
+        linear(x32 if x_run is None else x_run, self.w_x, None, low)
+        dt = torch.empty((tokens, self.inner), **f32)
+        linear(low[:, :self.rank], self.w_dt, None, dt)
+        y = self.runtime.empty((tokens, self.inner))
+        kernels.selective_scan(x32, dt, self.dt_b, low[:, self.rank:self.rank + self.states],
+                               low[:, self.rank + self.states:], self.a_log, self.skip, xz[:, self.inner:], state,
+                               batch.entry_start, batch.entry_first_pos, batch.slots, y, entries)
+        linear(y, self.w_o, None, residual, accumulate=accumulate)
+
+
 register_mixer("gated_delta", GatedDelta)
+register_mixer("decay_attention", DecayAttention)
+register_mixer("selective_scan", SelectiveScan)
 register_mixer("wkv", Wkv)

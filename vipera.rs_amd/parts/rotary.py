@@ -34,10 +34,14 @@ class RotaryNeox(PositionEncoding):
         self.head_dim = int(spec.params["head_dim"])
         self.rotary_dim = int(spec.params.get("rotary_dim", self.head_dim))
         self.base = float(spec.params["base"])
+        # linear scaling: every frequency divided by one factor (positions count as that much closer together)
+        self.scaling_factor = float(spec.params.get("scaling_factor") or 1.0)
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
             raise InvalidArgumentError(
                 f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
         table = neox_inverse_frequencies(self.rotary_dim, self.base)
+        if self.scaling_factor != 1.0:
+            table = (table / np.float32(self.scaling_factor)).astype(np.float32)
         self.inv_freq = torch.from_numpy(table).to(runtime.device)
 
     def fused_rotary(self):
@@ -48,7 +52,7 @@ class RotaryNeox(PositionEncoding):
         # again; a few decoded tokens are cheaper without the extra launch
         if batch.num_tokens < ANGLE_TABLE_MIN_TOKENS or not self.rotary_dim:
             return None
-        key = ("rope_angles", self.base, self.rotary_dim)
+        key = ("rope_angles", self.base, self.rotary_dim, self.scaling_factor)
         table = batch.shared.get(key)
         if table is None:
             table = batch.shared[key] = kernels.rope_angles(batch.positions, self.inv_freq, batch.num_tokens)
