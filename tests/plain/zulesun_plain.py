@@ -155,12 +155,31 @@ def route(scores, top, count, keep):
     return sorted(allowed, key=lambda e: (-scores[e], e))[:top]
 
 
-def moe(h, w, p):
+def routing_gap(z, top, count, keep):
+    """How far one token's router logits ``z`` are from another choice: the smallest difference between something
+    chosen (a kept group's best logit, a chosen expert's logit) and the best thing of its kind that was not."""
+    experts = z.shape[0]
+    size = experts // count
+    gap = np.inf
+    groups = np.sort(z.reshape(count, size).max(axis=1))[::-1]
+    if keep < count:
+        gap = min(gap, groups[keep - 1] - groups[keep])
+    chosen = route(z, top, count, keep)
+    best = sorted(range(count), key=lambda g: (-z.reshape(count, size).max(axis=1)[g], g))[:keep]
+    rest = [z[e] for e in range(experts) if e // size in best and e not in chosen]
+    if rest:
+        gap = min(gap, min(z[e] for e in chosen) - max(rest))
+    return gap
+
+
+def moe(h, w, p, gaps=None):
     router = p["router"]
     experts, top = router["experts"], router["top"]
     groups = router.get("groups") or {}
     count, keep = int(groups.get("count", 1)), int(groups.get("keep", groups.get("count", 1)))
     z = h @ w["router"].T
+    if gaps is not None:
+        gaps.append(np.array([routing_gap(z[t], top, count, keep) for t in range(h.shape[0])]))
     z = z - z.max(axis=-1, keepdims=True)
     scores = np.exp(z) / np.exp(z).sum(axis=-1, keepdims=True)
     out = np.zeros((h.shape[0], w["e0.down"].shape[0]))
@@ -183,8 +202,9 @@ def sub(weights, prefix):
     return {name[len(prefix):]: value for name, value in weights.items() if name.startswith(prefix)}
 
 
-def forward(config, weights, tokens, layers_out=None):
-    """Logits ``[tokens, vocab]`` of one sequence from position 0; ``layers_out`` collects the stream after each layer."""
+def forward(config, weights, tokens, layers_out=None, gaps=None):
+    """Logits ``[tokens, vocab]`` of one sequence from position 0; ``layers_out`` collects the stream after each layer,
+    ``gaps`` per mixture of experts every token's :func:`routing_gap`."""
     tokens = np.asarray(tokens)
     eps = float(config["norm"]["eps"])
     x = weights["embed"][tokens] * float(config["embedding"]["scale"])
@@ -202,7 +222,7 @@ def forward(config, weights, tokens, layers_out=None):
         mlp = layer.get("mlp")
         if mlp is not None:
             h = norm_around_zero(x, w["norm2"], eps)
-            y = dense_ffn(h, sub(w, "mlp.")) if mlp["kind"] == "dense" else moe(h, sub(w, "mlp."), mlp)
+            y = dense_ffn(h, sub(w, "mlp.")) if mlp["kind"] == "dense" else moe(h, sub(w, "mlp."), mlp, gaps)
             x = x + norm_around_zero(y, w["norm2b"], eps)
         if side:
             x = x + token_side(x, tokens, weights["side.embed"], index, sub(w, "side."), int(side["dim"]), eps)

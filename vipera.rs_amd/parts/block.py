@@ -141,6 +141,13 @@ class SandwichBlock(Block):
         out: List[TensorSpec] = []
         for _, family, part in cls._roles(spec):
             out += part_class(family, part.kind).declare(part, spec.prefix)
+        if spec.ffn.kind == "none":
+            # a layer without a feed-forward does not read the norms around it; a folder that stores them all the
+            # same is not refused for it
+            for norm in (spec.ffn_norm, spec.extras.get("ffn_post_norm")):
+                if norm is not None:
+                    out += [TensorSpec(t.name, t.shape, t.role, t.init, t.std, True)
+                            for t in part_class("norm", norm.kind).declare(norm, spec.prefix)]
         return out
 
     @classmethod
