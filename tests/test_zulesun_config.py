@@ -19,7 +19,7 @@ def test_the_architecture_is_found_by_its_name_and_layers_become_parts():
     specs = cfg.layer_specs()
     assert [s.mixer.kind for s in specs] == ["mixer_pair", "decay_attention", "mixer_pair", "decay_attention"]
     assert [s.ffn.kind for s in specs] == ["moe", "mlp", "none", "moe"]
-    assert all(s.block == "sandwich" and s.mixer_norm.params["one_plus"] for s in specs)
+    assert all(s.block == "sandwich_norm" and s.mixer_norm.params["one_plus"] for s in specs)
     assert all(s.extras["after"].kind == "token_side" and s.extras["after"].params["index"] == i for i, s in enumerate(specs))
     assert [s.position.kind for s in specs] == ["rotary_neox", "none", "rotary_neox", "none"]
     first = specs[0].mixer.params

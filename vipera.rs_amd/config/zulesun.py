@@ -235,7 +235,7 @@ class ZulesunConfig(ModelConfig):
             if self.side_dim:
                 extras["after"] = PartSpec("token_side", {"hidden": self.width, "dim": self.side_dim, "index": index,
                                                           "eps": self.eps, "activation": "gelu_tanh", "name": "side"})
-            specs.append(LayerSpec("sandwich", mixer, self._ffn(layer.get("mlp")), self._norm("norm1"),
+            specs.append(LayerSpec("sandwich_norm", mixer, self._ffn(layer.get("mlp")), self._norm("norm1"),
                                    self._norm("norm2"), position, f"l{index}.", extras))
         return specs
 

@@ -3,7 +3,7 @@
 ``prenorm``: ``x += mixer(norm_1(x)); x += ffn(norm_2(x))``, the pre-norm residual block of the
 reference (crates/vipera-backend-cpu/src/model.rs:3-4, 975-1198).
 ``parallel``: ``h = norm(x); x += mixer(h) + ffn(h)``.
-``sandwich``: a norm before and behind each sublayer, ``x += norm_1b(mixer(norm_1(x))); x += norm_2b(ffn(norm_2(x)))``,
+``sandwich_norm``: a norm before and behind each sublayer, ``x += norm_1b(mixer(norm_1(x))); x += norm_2b(ffn(norm_2(x)))``,
 and optionally a part that adds to the stream after both (``extras["after"]``, of the feed-forward family; it reads the
 32-bit stream itself).  The norms behind the sublayers are ``extras["mixer_post_norm"]`` and ``extras["ffn_post_norm"]``.
 """
@@ -183,5 +183,5 @@ class SandwichBlock(Block):
 
 
 register_block("prenorm", PreNormBlock)
-register_block("sandwich", SandwichBlock)
+register_block("sandwich_norm", SandwichBlock)
 register_block("parallel", ParallelBlock)
