@@ -106,7 +106,7 @@ def main() -> int:
                         help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
                              "pair of GPU events around every kernel launch, and add the microseconds of each class of "
                              "kernel to the line (split_decode_us, split_prefill_us)")
-    parser.add_argument("--design", default="", choices=["", "gilidra"],
+    parser.add_argument("--design", default="", choices=["", "gilidra", "zulesun"],
                         help="instead of the headline measurement: prefill and decode of this design at layer sizes that "
                              "resemble a real model's (--size), beside the dense Qwen2 decoder of the same width, depth and "
                              "active feed-forward width, each with the time of every class of kernel")
@@ -392,6 +392,31 @@ def gilidra_shape(z):
             "logit_scale": 1.0, "layers": layers}
 
 
+def zulesun_shape(z):
+    """A Zulesun configuration of sizes ``z``: linear attention with a decay per head, then twice attention over blocks
+    of positions beside a selective scan, and so on; a dense feed-forward in the first layer and a mixture of experts
+    chosen within groups in the others; a side table of 64 columns a layer."""
+    heads = z["heads"]
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": 4, "keep": 2}}}
+    lightning = {"heads": heads, "dim": z["dim"], "vdim": z["dim"],
+                 "decay": [1.0 - 2.0 ** (-1.0 - 7.0 * h / max(1, heads - 1)) for h in range(heads)]}
+    pair = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": z["dim"], "vdim": z["dim"],
+                     "mask": {"size": z["window"]}, "rot": {"base": 1e6, "dims": z["dim"] // 2, "scaling": {"factor": 8.0}},
+                     "scale": z["dim"] ** -0.5, "softcap": 30.0},
+            "left_scale": 1.0, "right_scale": 1.0,
+            "right": {"inner": 2 * z["width"], "state": 16, "dt_rank": z["width"] // 16, "conv": 4}}
+    layers = []
+    for index in range(z["layers"]):
+        mlp = {"kind": "dense", "ff": z["top"] * z["ff"]} if index == 0 else moe
+        if index % 5 in (0, 3):
+            layers.append({"type": "lightning", "mixer": lightning, "mlp": mlp})
+        else:
+            layers.append({"type": "parallel", "mixer": pair, "mlp": mlp})
+    return {"architecture": "Zulesun", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
+            "embedding": {"scale": z["width"] ** 0.5}, "token_side": {"dim": 64}, "layers": layers}
+
+
 def dense_shape(z):
     """The dense Qwen2 decoder of the same width, depth, heads and active feed-forward width."""
     return dict(QWEN25_7B, num_hidden_layers=z["layers"], hidden_size=z["width"], num_attention_heads=z["heads"],
@@ -420,7 +445,11 @@ def design_comparison(args) -> int:
     largest = max(batches)
     gen = torch.Generator().manual_seed(0)
     out = {}
-    for name, shape in (("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))):
+    # Gilidra beside the dense decoder; Zulesun beside Gilidra, the engine's other decoder of recurrences, attention
+    # over a part of the positions and mixtures of experts, and beside the dense decoder
+    runs = ((("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))) if args.design == "gilidra" else
+            (("zulesun", zulesun_shape(z)), ("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))))
+    for name, shape in runs:
         config = config_from_dict(shape)
         runtime = Runtime("cuda:0", args.dtype)
         model = build_model(config, runtime)
@@ -481,7 +510,8 @@ def design_comparison(args) -> int:
         out[name] = result
         del runner, model
         torch.cuda.empty_cache()
-    print(json.dumps({"metric": f"prefill and decode of {args.design} beside the dense decoder of equal size",
+    print(json.dumps({"metric": f"prefill and decode of {args.design} beside " + ("the dense decoder" if args.design == "gilidra"
+                                                                                    else "Gilidra and the dense decoder") + " of equal size",
                       "size": z, "dtype": args.dtype, "prefill_tokens": T, "ctx": ctx, "data": "synthetic: seeded random "
                       "weights and uniform-random token ids", **out}), flush=True)
     return 0
