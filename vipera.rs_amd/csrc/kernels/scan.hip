@@ -9,7 +9,7 @@
 // Both recurrences give the sixteen lanes of a quarter of a wave one output channel: each lane keeps R of the
 // channel's state numbers in registers, a sum over the state is R terms in a lane in ascending order and then four
 // exchanges inside the sixteen lanes.  That order depends on the sizes alone, so a token's result does not depend
-// on how its prompt was cut or on what else is in the step.  A workgroup owns sixteen channels of one entry and
+// on how its prompt was cut or on what else is in the step.  A workgroup (one wave) owns four channels of one entry and
 // walks the entry's tokens in order; the next token's operands are requested before the current one is worked on,
 // and no load sits behind a branch (a token past the entry's end reads the last one again).
 #include "common.h"
@@ -18,13 +18,24 @@ __device__ __forceinline__ float scan_silu(float z) { return z / (1.0f + expf(-z
 __device__ __forceinline__ float scan_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float scan_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 
+template <int CTRL>
+__device__ __forceinline__ float scan_dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
+  return v + __int_as_float(moved);
+}
+
+// The sum over the 16 lanes of a row, in every lane, without LDS: neighbours, pairs of neighbours, the other quad of
+// the eight, the other eight.
 __device__ __forceinline__ float row16_sum(float v) {
-  v += __shfl_xor(v, 1, WAVE);
-  v += __shfl_xor(v, 2, WAVE);
-  v += __shfl_xor(v, 4, WAVE);
-  v += __shfl_xor(v, 8, WAVE);
+  v = scan_dpp_add<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  v = scan_dpp_add<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  v = scan_dpp_add<0x141>(v);    // row_half_mirror
+  v = scan_dpp_add<0x140>(v);    // row_mirror
   return v;
 }
+
+constexpr int SCAN_THREADS = 64;      // a workgroup is one wave: four channels of sixteen lanes
+constexpr int SCAN_CHANNELS = 4;
 
 static inline int lanes_share(int n) { return n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 4 : n <= 128 ? 8 : 16; }
 
@@ -33,9 +44,10 @@ static inline int lanes_share(int n) { return n <= 16 ? 1 : n <= 32 ? 2 : n <= 6
 //   q, k  [T, ldqk] 32-bit, head h at columns h * dim;  v [T, ldv], head h at columns h * vdim
 //   act   1: q, k and v pass through silu as they are read
 //   state per head `vdim * 16 R` floats: value channel c holds its key channels, padded to 16 R, one after another
-// Grid (entries, heads, ceil(vdim / 16)).
-template <int R>
-__global__ __launch_bounds__(256) void decay_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
+// Grid (entries, heads, ceil(vdim / 4)).  VEC: dim = 16 R with R a multiple of 4 and 16-byte rows, so a lane's run of
+// key channels is read four at a time.
+template <int R, bool VEC>
+__global__ __launch_bounds__(SCAN_THREADS) void decay_rule_kernel(const float* __restrict__ q, const float* __restrict__ k,
                                                          long long ldqk, const float* __restrict__ v, long long ldv,
                                                          int act, const float* __restrict__ decay,
                                                          float* __restrict__ state, long long state_stride,
@@ -44,9 +56,9 @@ __global__ __launch_bounds__(256) void decay_rule_kernel(const float* __restrict
                                                          const int* __restrict__ slots, int heads, int dim, int vdim,
                                                          float* __restrict__ o) {
   const int e = blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
   const int part = lane & 15;
-  const int vch = blockIdx.z * 16 + wave * 4 + (lane >> 4);
+  const int vch = blockIdx.z * SCAN_CHANNELS + (lane >> 4);
   const bool live = vch < vdim;
   const int vcol = h * vdim + min(vch, vdim - 1);
   const int t0 = entry_start[e], t1 = entry_start[e + 1];
@@ -65,53 +77,72 @@ __global__ __launch_bounds__(256) void decay_rule_kernel(const float* __restrict
     s[r] = (fresh || !in[r]) ? 0.f : old;
   }
   if (t1 <= t0) return;
-  float nk[R], nq[R], nv;
-  {
-    const float* kr = k + (long long)t0 * ldqk;
-    const float* qr = q + (long long)t0 * ldqk;
+  // D tokens' operands are on their way while the D before them are worked on: a token's step is a few dozen
+  // instructions, a load's way through the caches several hundred cycles
+  constexpr int D = R >= 16 ? 2 : 4;
+  float nk[D][R], nq[D][R], nv[D];
+  auto fetch = [&](int first) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      nk[r] = kr[col[r]];
-      nq[r] = qr[col[r]];
-    }
-    nv = v[(long long)t0 * ldv + vcol];
-  }
-  for (int t = t0; t < t1; ++t) {
-    float ck[R], cq[R];
+    for (int j = 0; j < D; ++j) {
+      const int t = min(first + j, t1 - 1);
+      const float* kr = k + (long long)t * ldqk;
+      const float* qr = q + (long long)t * ldqk;
+      if constexpr (VEC) {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      ck[r] = nk[r];
-      cq[r] = nq[r];
+        for (int r = 0; r < R; r += 4) {
+          const f32x4 k4 = *(const f32x4*)(kr + col[r]), q4 = *(const f32x4*)(qr + col[r]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            nk[j][r + i] = k4[i];
+            nq[j][r + i] = q4[i];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          nk[j][r] = kr[col[r]];
+          nq[j][r] = qr[col[r]];
+        }
+      }
+      nv[j] = v[(long long)t * ldv + vcol];
     }
-    float cv = nv;
-    const int tn = min(t + 1, t1 - 1);
-    {
-      const float* kr = k + (long long)tn * ldqk;
-      const float* qr = q + (long long)tn * ldqk;
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += D) {
+    float ck[D][R], cq[D][R], cv[D];
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        nk[r] = kr[col[r]];
-        nq[r] = qr[col[r]];
+        ck[j][r] = nk[j][r];
+        cq[j][r] = nq[j][r];
       }
-      nv = v[(long long)tn * ldv + vcol];
+      cv[j] = nv[j];
     }
-    if (act) {
+    fetch(tb + D);
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+      const int t = tb + j;
+      if (t >= t1) break;
+      if (act) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          ck[j][r] = scan_silu(ck[j][r]);
+          cq[j][r] = scan_silu(cq[j][r]);
+        }
+        cv[j] = scan_silu(cv[j]);
+      }
+      float sum = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        ck[r] = scan_silu(ck[r]);
-        cq[r] = scan_silu(cq[r]);
+        const float kk = in[r] ? ck[j][r] : 0.f;
+        s[r] = fmaf(rate, s[r], kk * cv[j]);
+        sum = fmaf(s[r], in[r] ? cq[j][r] : 0.f, sum);
       }
-      cv = scan_silu(cv);
+      sum = row16_sum(sum);
+      if (part == 0 && live) o[(long long)t * heads * vdim + vcol] = sum;
     }
-    float sum = 0.f;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const float kk = in[r] ? ck[r] : 0.f;
-      s[r] = fmaf(rate, s[r], kk * cv);
-      sum = fmaf(s[r], in[r] ? cq[r] : 0.f, sum);
-    }
-    sum = row16_sum(sum);
-    if (part == 0 && live) o[(long long)t * heads * vdim + vcol] = sum;
   }
   if (live) {
 #pragma unroll
@@ -129,18 +160,20 @@ extern "C" int vk_decay_rule(const float* q, const float* k, long long ldqk, con
   if (heads < 1 || dim < 1 || vdim < 1 || heads > 65535) return VK_BAD_ARGUMENT;
   if (dim > 256) return VK_UNSUPPORTED_SIZE;
   if (state_stride < heads * vk_decay_rule_head_floats(dim, vdim)) return VK_BAD_ARGUMENT;
-  dim3 grid(num_entries, heads, (vdim + 15) / 16);
+  dim3 grid(num_entries, heads, (vdim + SCAN_CHANNELS - 1) / SCAN_CHANNELS);
   if (grid.z > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-#define VK_DR(RR)                                                                                                  \
-  decay_rule_kernel<RR><<<grid, 256, 0, s>>>(q, k, ldqk, v, ldv, act, decay, state, state_stride, entry_start,     \
-                                             entry_first, slots, heads, dim, vdim, o)
-  switch (lanes_share(dim)) {
-    case 1: VK_DR(1); break;
-    case 2: VK_DR(2); break;
-    case 4: VK_DR(4); break;
-    case 8: VK_DR(8); break;
-    default: VK_DR(16); break;
+  const int share = lanes_share(dim);
+  const bool vec = share >= 4 && dim == 16 * share && ldqk % 4 == 0 && (((uintptr_t)q | (uintptr_t)k) & 15) == 0;
+#define VK_DR(RR, VV)                                                                                                 \
+  decay_rule_kernel<RR, VV><<<grid, SCAN_THREADS, 0, s>>>(q, k, ldqk, v, ldv, act, decay, state, state_stride,        \
+                                                          entry_start, entry_first, slots, heads, dim, vdim, o)
+  switch (share) {
+    case 1: VK_DR(1, false); break;
+    case 2: VK_DR(2, false); break;
+    case 4: if (vec) VK_DR(4, true); else VK_DR(4, false); break;
+    case 8: if (vec) VK_DR(8, true); else VK_DR(8, false); break;
+    default: if (vec) VK_DR(16, true); else VK_DR(16, false); break;
   }
 #undef VK_DR
   VK_LAUNCH_CHECK();
@@ -277,18 +310,20 @@ extern "C" int vk_causal_conv(const float* in, long long ldi, const float* conv,
 //   y = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])
 //   A = -exp(a_log) [C, N];  B and C are column ranges of one [T, ldbc] buffer;  z a column range of [T, ldz]
 //   state per channel 16 R floats (N padded), channel after channel
-// Grid (entries, ceil(C / 16)).
+//   prepared: dtraw already holds softplus(dt + dt_bias) and z already silu(z) (scan_prepare below; a prompt's tokens
+//   would each pay for them behind one another here)
+// Grid (entries, ceil(C / 4)).
 template <int R, typename TO>
-__global__ __launch_bounds__(256) void selective_scan_kernel(
+__global__ __launch_bounds__(SCAN_THREADS) void selective_scan_kernel(
     const float* __restrict__ x, const float* __restrict__ dtraw, long long lddt, const float* __restrict__ dt_bias,
     const float* __restrict__ bmat, const float* __restrict__ cmat, long long ldbc, const float* __restrict__ a_log,
     const float* __restrict__ skip, const float* __restrict__ z, long long ldz, float* __restrict__ state,
     long long state_stride, const int* __restrict__ entry_start, const int* __restrict__ entry_first,
-    const int* __restrict__ slots, int C, int N, TO* __restrict__ out) {
+    const int* __restrict__ slots, int C, int N, int prepared, TO* __restrict__ out) {
   const int e = blockIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
   const int part = lane & 15;
-  const int ch_raw = blockIdx.y * 16 + wave * 4 + (lane >> 4);
+  const int ch_raw = blockIdx.y * SCAN_CHANNELS + (lane >> 4);
   const bool live = ch_raw < C;
   const int ch = min(ch_raw, C - 1);
   const int t0 = entry_start[e], t1 = entry_start[e + 1];
@@ -308,52 +343,84 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
   }
   if (t1 <= t0) return;
   const float bias = dt_bias[ch], d = skip[ch];
-  float nb[R], nc[R], nx, ndt, nz;
-  {
+  // D tokens' operands are on their way while the D before them are worked on (see decay_rule_kernel)
+  constexpr int D = R >= 8 ? 2 : R >= 4 ? 4 : 8;
+  float nb[D][R], nc[D][R], nx[D], ndt[D], nz[D];
+  auto fetch = [&](int first) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      nb[r] = bmat[(long long)t0 * ldbc + col[r]];
-      nc[r] = cmat[(long long)t0 * ldbc + col[r]];
-    }
-    nx = x[(long long)t0 * C + ch];
-    ndt = dtraw[(long long)t0 * lddt + ch];
-    nz = z[(long long)t0 * ldz + ch];
-  }
-  for (int t = t0; t < t1; ++t) {
-    float cb[R], cc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      cb[r] = nb[r];
-      cc[r] = nc[r];
-    }
-    const float cx = nx, cdt = ndt, cz = nz;
-    const int tn = min(t + 1, t1 - 1);
-    {
+    for (int j = 0; j < D; ++j) {
+      const int t = min(first + j, t1 - 1);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        nb[r] = bmat[(long long)tn * ldbc + col[r]];
-        nc[r] = cmat[(long long)tn * ldbc + col[r]];
+        nb[j][r] = bmat[(long long)t * ldbc + col[r]];
+        nc[j][r] = cmat[(long long)t * ldbc + col[r]];
       }
-      nx = x[(long long)tn * C + ch];
-      ndt = dtraw[(long long)tn * lddt + ch];
-      nz = z[(long long)tn * ldz + ch];
+      nx[j] = x[(long long)t * C + ch];
+      ndt[j] = dtraw[(long long)t * lddt + ch];
+      nz[j] = z[(long long)t * ldz + ch];
     }
-    const float dt = scan_softplus(cdt + bias);
-    const float dtx = dt * cx;
-    float sum = 0.f;
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += D) {
+    float cb[D][R], cc[D][R], cx[D], cdt[D], cz[D];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const float keep = expf(dt * a[r]);
-      s[r] = fmaf(keep, s[r], in[r] ? dtx * cb[r] : 0.f);
-      sum = fmaf(s[r], in[r] ? cc[r] : 0.f, sum);
+    for (int j = 0; j < D; ++j) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        cb[j][r] = nb[j][r];
+        cc[j][r] = nc[j][r];
+      }
+      cx[j] = nx[j];
+      cdt[j] = ndt[j];
+      cz[j] = nz[j];
     }
-    sum = row16_sum(sum);
-    if (part == 0 && live) out[(long long)t * C + ch] = from_float<TO>(fmaf(d, cx, sum) * scan_silu(cz));
+    fetch(tb + D);
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+      const int t = tb + j;
+      if (t >= t1) break;
+      const float dt = prepared ? cdt[j] : scan_softplus(cdt[j] + bias);
+      const float dtx = dt * cx[j];
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float keep = expf(dt * a[r]);
+        s[r] = fmaf(keep, s[r], in[r] ? dtx * cb[j][r] : 0.f);
+        sum = fmaf(s[r], in[r] ? cc[j][r] : 0.f, sum);
+      }
+      sum = row16_sum(sum);
+      if (part == 0 && live)
+        out[(long long)t * C + ch] = from_float<TO>(fmaf(d, cx[j], sum) * (prepared ? cz[j] : scan_silu(cz[j])));
+    }
   }
   if (live) {
 #pragma unroll
     for (int r = 0; r < R; ++r) row[r] = s[r];
   }
+}
+
+// dt[t, c] <- softplus(dt[t, c] + dt_bias[c]) in place and gate[t, c] = silu(z[t, c]): what the scan of a prompt's
+// portion would otherwise compute token behind token.
+__global__ void scan_prepare_kernel(float* __restrict__ dt, long long lddt, const float* __restrict__ dt_bias,
+                                    const float* __restrict__ z, long long ldz, float* __restrict__ gate, int C,
+                                    long long total) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long t = idx / C;
+  const int c = (int)(idx % C);
+  dt[t * lddt + c] = scan_softplus(dt[t * lddt + c] + dt_bias[c]);
+  gate[idx] = scan_silu(z[t * ldz + c]);
+}
+
+extern "C" int vk_scan_prepare(float* dt, long long lddt, const float* dt_bias, const float* z, long long ldz,
+                               float* gate, int num_tokens, int C, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (C < 1) return VK_BAD_ARGUMENT;
+  const long long total = (long long)num_tokens * C;
+  scan_prepare_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(dt, lddt, dt_bias, z, ldz, gate,
+                                                                                       C, total);
+  VK_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" long long vk_selective_scan_channel_floats(int states) { return 16LL * lanes_share(states); }
@@ -362,19 +429,19 @@ extern "C" int vk_selective_scan(const float* x, const float* dtraw, long long l
                                  const float* bmat, const float* cmat, long long ldbc, const float* a_log,
                                  const float* skip, const float* z, long long ldz, float* state,
                                  long long state_stride, const int* entry_start, const int* entry_first,
-                                 const int* slots, int num_entries, int C, int N, void* out, int out_dtype,
-                                 void* stream) {
+                                 const int* slots, int num_entries, int C, int N, int prepared, void* out,
+                                 int out_dtype, void* stream) {
   if (num_entries <= 0) return 0;
   if (C < 1 || N < 1) return VK_BAD_ARGUMENT;
   if (N > 256) return VK_UNSUPPORTED_SIZE;
   if (state_stride < (long long)C * vk_selective_scan_channel_floats(N)) return VK_BAD_ARGUMENT;
-  dim3 grid(num_entries, (C + 15) / 16);
+  dim3 grid(num_entries, (C + SCAN_CHANNELS - 1) / SCAN_CHANNELS);
   if (grid.y > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
 #define VK_SS(RR, TO)                                                                                               \
-  selective_scan_kernel<RR, TO><<<grid, 256, 0, s>>>(x, dtraw, lddt, dt_bias, bmat, cmat, ldbc, a_log, skip, z, ldz, \
-                                                     state, state_stride, entry_start, entry_first, slots, C, N,    \
-                                                     (TO*)out)
+  selective_scan_kernel<RR, TO><<<grid, SCAN_THREADS, 0, s>>>(x, dtraw, lddt, dt_bias, bmat, cmat, ldbc, a_log, skip, \
+                                                              z, ldz, state, state_stride, entry_start, entry_first, \
+                                                              slots, C, N, prepared, (TO*)out)
 #define VK_SS_R(TO)                       \
   switch (lanes_share(N)) {               \
     case 1: VK_SS(1, TO); break;          \

@@ -1379,11 +1379,12 @@ def causal_conv(x: torch.Tensor, conv: torch.Tensor, bias: Optional[torch.Tensor
 def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, b: torch.Tensor, c: torch.Tensor,
                    a_log: torch.Tensor, skip: torch.Tensor, z: torch.Tensor, state: torch.Tensor,
                    entry_start: torch.Tensor, entry_first_pos: torch.Tensor, slots: torch.Tensor, out: torch.Tensor,
-                   num_entries: int) -> None:
+                   num_entries: int, prepared: bool = False) -> None:
     """The selective scan over the step's entries in 32-bit: per channel ``c`` and state ``n``
     ``step = softplus(dt + dt_bias); S <- exp(step * -exp(a_log)) S + step x b; y = S . c + skip x``, and
     ``out = y * silu(z)``.  ``x [T, C]`` contiguous; ``dt``, ``z`` row-strided views ``[T, C]``; ``b`` and ``c``
-    row-strided views ``[T, N]`` of one buffer; ``state`` starts with ``C * selective_scan_channel_floats(N)`` floats."""
+    row-strided views ``[T, N]`` of one buffer; ``state`` starts with ``C * selective_scan_channel_floats(N)`` floats.
+    ``prepared``: ``dt`` already holds ``softplus(dt + dt_bias)`` and ``z`` already ``silu(z)`` (:func:`scan_prepare`)."""
     _dev(x, dt, dt_bias, b, c, a_log, skip, z, state, entry_start, entry_first_pos, slots, out)
     tokens, channels = x.shape
     states = a_log.shape[1]
@@ -1404,7 +1405,23 @@ def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, b: 
     _i32(entry_start, entry_first_pos, slots)
     _entries_ok((entry_start, entry_first_pos, slots), num_entries)
     fn = _fn("scan", "vk_selective_scan", [_p, _p, _ll, _p, _p, _p, _ll, _p, _p, _p, _ll, _p, _ll, _p, _p, _p, _i, _i, _i,
-                                           _p, _i, _p])
+                                           _i, _p, _i, _p])
     _status(fn(_ptr(x), _ptr(dt), dt.stride(0), _ptr(dt_bias), _ptr(b), _ptr(c), b.stride(0), _ptr(a_log), _ptr(skip),
                _ptr(z), z.stride(0), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first_pos), _ptr(slots),
-               num_entries, channels, states, _ptr(out), _dt(out, "out"), _stream()), "selective_scan")
+               num_entries, channels, states, 1 if prepared else 0, _ptr(out), _dt(out, "out"), _stream()),
+            "selective_scan")
+
+
+def scan_prepare(dt: torch.Tensor, dt_bias: torch.Tensor, z: torch.Tensor, gate: torch.Tensor) -> None:
+    """``dt <- softplus(dt + dt_bias)`` in place and ``gate = silu(z)``, for :func:`selective_scan` with ``prepared``: a
+    prompt's portion takes them once for all its tokens instead of token behind token inside the recurrence."""
+    _dev(dt, dt_bias, z, gate)
+    tokens, channels = gate.shape
+    for t, what in ((dt, "dt"), (z, "z")):
+        _f32s(t, "scan_prepare: " + what)
+        _need(t.shape == gate.shape, "scan_prepare: shapes")
+    _f32(gate, "scan_prepare: gate")
+    _need(dt_bias.dtype == torch.float32 and dt_bias.numel() == channels and dt_bias.is_contiguous(), "scan_prepare: dt_bias")
+    fn = _fn("scan", "vk_scan_prepare", [_p, _ll, _p, _p, _ll, _p, _i, _i, _p])
+    _status(fn(_ptr(dt), dt.stride(0), _ptr(dt_bias), _ptr(z), z.stride(0), _ptr(gate), tokens, channels, _stream()),
+            "scan_prepare")

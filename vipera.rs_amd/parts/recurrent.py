@@ -268,7 +268,16 @@ class DecayAttention(Mixer):
         q, k = proj[:, :self.qk], proj[:, self.qk:2 * self.qk]
         v, g = proj[:, 2 * self.qk:2 * self.qk + self.vw], proj[:, 2 * self.qk + self.vw:]
         o = torch.empty((tokens, self.vw), **f32)
-        kernels.decay_rule(q, k, v, self.activation == "silu", self.decay, state, batch.entry_start,
+        inside = self.activation == "silu"
+        if inside and not batch.all_single:
+            # every workgroup of value channels would take the activation of a token's q and k again, token behind
+            # token: a prompt's portion takes it once, ahead of the recurrence; a step of single tokens saves the launch
+            width = 2 * self.qk + self.vw
+            ready = torch.empty((tokens, width), **f32)
+            kernels.activation(proj[:, :width], "silu", ready)
+            q, k, v = ready[:, :self.qk], ready[:, self.qk:2 * self.qk], ready[:, 2 * self.qk:]
+            inside = False
+        kernels.decay_rule(q, k, v, inside, self.decay, state, batch.entry_start,
                            batch.entry_first_pos, batch.slots, self.heads, self.dim, self.vdim, o, entries)
         gated = self.runtime.empty((tokens, self.vw))
         kernels.gated_norm(o, self.norm, g, self.gate, self.eps, gated)
@@ -339,9 +348,15 @@ class SelectiveScan(Mixer):
         dt = torch.empty((tokens, self.inner), **f32)
         linear(low[:, :self.rank], self.w_dt, None, dt)
         y = self.runtime.empty((tokens, self.inner))
+        z = xz[:, self.inner:]
+        ahead = not batch.all_single
+        if ahead:   # a prompt's portion: the step sizes' softplus and the gate's silu once, ahead of the recurrence
+            gate = torch.empty((tokens, self.inner), **f32)
+            kernels.scan_prepare(dt, self.dt_b, z, gate)
+            z = gate
         kernels.selective_scan(x32, dt, self.dt_b, low[:, self.rank:self.rank + self.states],
-                               low[:, self.rank + self.states:], self.a_log, self.skip, xz[:, self.inner:], state,
-                               batch.entry_start, batch.entry_first_pos, batch.slots, y, entries)
+                               low[:, self.rank + self.states:], self.a_log, self.skip, z, state,
+                               batch.entry_start, batch.entry_first_pos, batch.slots, y, entries, prepared=ahead)
         linear(y, self.w_o, None, residual, accumulate=accumulate)
 
 
