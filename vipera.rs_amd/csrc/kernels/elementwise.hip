@@ -517,8 +517,13 @@ extern "C" int vk_scale(float* x, float factor, long long count, void* stream) {
 // ---------------------------------------------------------------------------------------------
 // A norm behind a sublayer: residual[r, :] += y[r, :] / sqrt(mean(y[r, :]^2) + eps) * weight, all 32-bit.
 // One workgroup per row; the sum of squares in the order of `rmsnorm_kernel`'s general path.
+// With `next_out`: the new rows of the residual also leave as the input of what follows, in that part's type: normed
+// again (`next_weight`, `next_eps`: the norm in front of the next sublayer) or as they are (`next_weight` null).
+template <typename TO>
 __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restrict__ y, const float* __restrict__ weight,
-                                                          float* __restrict__ residual, int width, float eps) {
+                                                          float* __restrict__ residual, int width, float eps,
+                                                          const float* __restrict__ next_weight, float next_eps,
+                                                          TO* __restrict__ next_out) {
   __shared__ float scratch[16];
   const float* src = y + (size_t)blockIdx.x * width;
   float* dst = residual + (size_t)blockIdx.x * width;
@@ -529,14 +534,36 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restric
   }
   sum = block_sum(sum, scratch);
   const float inv = 1.0f / sqrtf(sum / (float)width + eps);
-  for (int i = threadIdx.x; i < width; i += 256) dst[i] += src[i] * inv * weight[i];
+  float again = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float x = dst[i] + src[i] * inv * weight[i];
+    dst[i] = x;
+    again += x * x;
+  }
+  if (next_out == nullptr) return;
+  TO* out = next_out + (size_t)blockIdx.x * width;
+  if (next_weight == nullptr) {
+    for (int i = threadIdx.x; i < width; i += 256) out[i] = from_float<TO>(dst[i]);   // a thread reads what it wrote
+    return;
+  }
+  again = block_sum(again, scratch);
+  const float next_inv = 1.0f / sqrtf(again / (float)width + next_eps);
+  for (int i = threadIdx.x; i < width; i += 256) out[i] = from_float<TO>(dst[i] * next_inv * next_weight[i]);
 }
 
 extern "C" int vk_rmsnorm_add(const float* y, const float* weight, float* residual, int num_rows, int width, float eps,
-                              void* stream) {
+                              const float* next_weight, float next_eps, void* next_out, int next_dtype, void* stream) {
   if (num_rows <= 0) return 0;
   if (width <= 0) return VK_BAD_ARGUMENT;
-  rmsnorm_add_kernel<<<num_rows, 256, 0, (hipStream_t)stream>>>(y, weight, residual, width, eps);
+  hipStream_t s = (hipStream_t)stream;
+  if (next_out == nullptr || next_dtype == DT_F32)
+    rmsnorm_add_kernel<float><<<num_rows, 256, 0, s>>>(y, weight, residual, width, eps, next_weight, next_eps,
+                                                       (float*)next_out);
+  else if (next_dtype == DT_BF16)
+    rmsnorm_add_kernel<bf16_t><<<num_rows, 256, 0, s>>>(y, weight, residual, width, eps, next_weight, next_eps,
+                                                        (bf16_t*)next_out);
+  else
+    return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
   return 0;
 }

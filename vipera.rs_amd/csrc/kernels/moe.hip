@@ -345,16 +345,16 @@ __global__ __launch_bounds__(256) void moe_down_mma_kernel(const __bf16* __restr
   }
 }
 
-// residual[t, :] += sum_j weights[t, j] * pair_out[t * top + j, :], j ascending.
+// residual[t, :] (+)= sum_j weights[t, j] * pair_out[t * top + j, :], j ascending.
 __global__ void moe_combine_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, int top,
-                                   int width, long long total, float* __restrict__ residual) {
+                                   int width, long long total, float* __restrict__ residual, int accumulate) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const long long t = idx / width;
   const int c = (int)(idx % width);
   float sum = 0.f;
   for (int j = 0; j < top; ++j) sum = fmaf(weights[t * top + j], pair_out[(t * top + j) * width + c], sum);
-  residual[idx] += sum;
+  residual[idx] = accumulate ? residual[idx] + sum : sum;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -403,10 +403,12 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
                               num_tiles, stream);
 }
 
-extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
-                              const int* offsets, const int* order, const int* tiles, const int* num_tiles,
-                              const float* weights, int num_tokens, int experts, int top, int width, int ff,
-                              float limit, float alpha, void* act, float* pair_out, float* residual, void* stream) {
+// accumulate 0: the weighted sums are written to `residual` instead of added to it.
+extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
+                                   const int* offsets, const int* order, const int* tiles, const int* num_tiles,
+                                   const float* weights, int num_tokens, int experts, int top, int width, int ff,
+                                   float limit, float alpha, void* act, float* pair_out, float* residual,
+                                   int accumulate, void* stream) {
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || width < 1 || ff < 1) return VK_BAD_ARGUMENT;
   const int pairs = num_tokens * top;
@@ -431,7 +433,7 @@ extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, cons
                                                         num_tiles, width, ff, pair_out);
     VK_LAUNCH_CHECK();
     const long long all = (long long)num_tokens * width;
-    moe_combine_kernel<<<(unsigned)((all + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, all, residual);
+    moe_combine_kernel<<<(unsigned)((all + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, all, residual, accumulate);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -457,7 +459,15 @@ extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, cons
   }
   VK_LAUNCH_CHECK();
   const long long total = (long long)num_tokens * width;
-  moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, total, residual);
+  moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, total, residual, accumulate);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
+                              const int* offsets, const int* order, const int* tiles, const int* num_tiles,
+                              const float* weights, int num_tokens, int experts, int top, int width, int ff,
+                              float limit, float alpha, void* act, float* pair_out, float* residual, void* stream) {
+  return vk_moe_experts_into(h, ldh, wg, wu, wd, dtype, offsets, order, tiles, num_tiles, weights, num_tokens, experts,
+                             top, width, ff, limit, alpha, act, pair_out, residual, 1, stream);
 }

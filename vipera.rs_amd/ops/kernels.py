@@ -1169,10 +1169,11 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
 
 def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
                 order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, weights: torch.Tensor, top: int,
-                limit: float, alpha: float, act: torch.Tensor, pair_out: torch.Tensor, residual: torch.Tensor) -> None:
+                limit: float, alpha: float, act: torch.Tensor, pair_out: torch.Tensor, residual: torch.Tensor,
+                accumulate: bool = True) -> None:
     """The chosen experts of every token: ``y = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(Wg h, limit)`` and
     ``u = clamp(Wu h, -limit, limit)``, or with an infinite ``limit`` ``y = g * sigmoid(alpha * g) * u`` (alpha 1:
-    ``silu(g) * u``); then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])``."""
+    ``silu(g) * u``); then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])`` (without ``accumulate``: ``=``)."""
     _dev(h, w_gate, w_up, w_down, offsets, order, tiles, num_tiles, weights, act, pair_out, residual)
     tokens, width = h.shape
     experts, ff, _ = w_gate.shape
@@ -1190,10 +1191,11 @@ def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_dow
     _need(offsets.numel() == experts + 1 and order.numel() == tokens * top
           and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts, moe_tile_rows(h, width, ff)),
           "moe_experts: grouping (made by moe_route with moe_tile_rows(h, width, ff))")
-    fn = _fn("moe", "vk_moe_experts", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p, _p, _p])
+    fn = _fn("moe", "vk_moe_experts_into", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p, _p,
+                                            _i, _p])
     _status(fn(_ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _dt(h, "h"), _ptr(offsets), _ptr(order),
                _ptr(tiles), _ptr(num_tiles), _ptr(weights), tokens, experts, top, width, ff, float(limit), float(alpha),
-               _ptr(act), _ptr(pair_out), _ptr(residual), _stream()), "moe_experts")
+               _ptr(act), _ptr(pair_out), _ptr(residual), 1 if accumulate else 0, _stream()), "moe_experts")
 
 
 # --- norms behind a sublayer, sums of two streams, activations ------------------------------------------
@@ -1202,16 +1204,26 @@ def _f32s(tensor: torch.Tensor, what: str) -> None:
     _need(tensor.dtype == torch.float32 and tensor.stride(-1) == 1, f"{what} must be float32 with a unit inner stride")
 
 
-def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor) -> None:
-    """``residual += y / sqrt(mean(y^2) + eps) * weight`` row by row, all 32-bit."""
-    _dev(y, weight, residual)
+def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor,
+                next_out: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
+                next_eps: float = 0.0) -> None:
+    """``residual += y / sqrt(mean(y^2) + eps) * weight`` row by row, all 32-bit.  With ``next_out`` the new rows also
+    leave as the next part's input, in its dtype: ``residual / sqrt(mean(residual^2) + next_eps) * next_weight`` (the
+    norm in front of the next sublayer), or the rows as they are without ``next_weight``."""
+    _dev(y, weight, residual, next_out, next_weight)
     _f32(y, "rmsnorm_add: y")
     _f32(residual, "rmsnorm_add: residual")
     rows, width = residual.shape
     _need(y.shape == residual.shape and y.is_contiguous() and residual.is_contiguous(), "rmsnorm_add: shapes")
     _need(weight.dtype == torch.float32 and weight.numel() == width and weight.is_contiguous(), "rmsnorm_add: weight")
-    fn = _fn("elementwise", "vk_rmsnorm_add", [_p, _p, _p, _i, _i, _f, _p])
-    _status(fn(_ptr(y), _ptr(weight), _ptr(residual), rows, width, float(eps), _stream()), "rmsnorm_add")
+    if next_out is not None:
+        _need(next_out.shape == residual.shape and next_out.is_contiguous(), "rmsnorm_add: next_out")
+    if next_weight is not None:
+        _need(next_out is not None and next_weight.dtype == torch.float32 and next_weight.numel() == width
+              and next_weight.is_contiguous(), "rmsnorm_add: next_weight")
+    fn = _fn("elementwise", "vk_rmsnorm_add", [_p, _p, _p, _i, _i, _f, _p, _f, _p, _i, _p])
+    _status(fn(_ptr(y), _ptr(weight), _ptr(residual), rows, width, float(eps), _ptr(next_weight), float(next_eps),
+               _ptr(next_out), _dt(next_out, "next_out") if next_out is not None else 0, _stream()), "rmsnorm_add")
 
 
 def axpby(x: torch.Tensor, a: float, y: torch.Tensor, b: float, out: torch.Tensor, accumulate: bool = False) -> None:

@@ -120,8 +120,10 @@ class Norm(Part):
         """A :class:`NormHandoff` for ``tokens`` rows if this norm can be split between its neighbours, else None."""
         return None
 
-    def add_into(self, y: torch.Tensor, residual: torch.Tensor) -> None:
-        """``residual += norm(y)`` in 32-bit: what a block calls for a norm that stands behind a sublayer."""
+    def add_into(self, y: torch.Tensor, residual: torch.Tensor, follow=None, as_input: bool = False):
+        """``residual += norm(y)`` in 32-bit: what a block calls for a norm that stands behind a sublayer.  With
+        ``follow`` (the norm in front of the next sublayer) it returns that norm's output of the new rows; with
+        ``as_input`` the new rows in the run's dtype; else None."""
         raise NotImplementedError
 
 

@@ -169,17 +169,21 @@ class SandwichBlock(Block):
         else:
             y = torch.zeros_like(x)
             parts["mixer"].forward(h, batch, cache, state, parts["position"], y, reads_only)
-        parts["mixer_post_norm"].add_into(y, x)
-        if self.has_ffn:
-            h = parts["ffn_norm"].forward(x)
+        after = parts.get("after")
+        feeds_after = after is not None and getattr(after, "reads_stream_input", False)
+        if not self.has_ffn:
+            stream = parts["mixer_post_norm"].add_into(y, x, as_input=feeds_after)
+        else:
+            # the norm behind the mixer and the one in front of the feed-forward: one launch where both are of a kind
+            h = parts["mixer_post_norm"].add_into(y, x, follow=parts["ffn_norm"])
             if parts["ffn"].can_overwrite:
                 parts["ffn"].forward(h, batch, y, accumulate=False)
             else:
                 y.zero_()
                 parts["ffn"].forward(h, batch, y)
-            parts["ffn_post_norm"].add_into(y, x)
-        if "after" in parts:
-            parts["after"].forward(None, batch, x)
+            stream = parts["ffn_post_norm"].add_into(y, x, as_input=feeds_after)
+        if after is not None:
+            after.forward(stream if feeds_after else None, batch, x)
 
 
 register_block("prenorm", PreNormBlock)

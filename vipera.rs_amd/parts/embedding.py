@@ -99,8 +99,11 @@ class Embedding(Part):
 class TokenSide(FeedForward):
     """What a layer adds to the stream from its own columns of the per-token side table (see :class:`Embedding`):
     ``e = side[token][index * dim : (index + 1) * dim]``, ``g = gelu_tanh(Wgate x) * e``, ``y = Wproj g``,
-    ``x += y / rms(y) * norm``.  It reads the 32-bit stream ``x`` itself (``h`` is not used).  ``params``: ``hidden``,
+    ``x += y / rms(y) * norm``.  It reads the stream ``x`` itself: ``h`` is the stream in the run's dtype if the block
+    has it at hand (``reads_stream_input``), else it is made here.  ``params``: ``hidden``,
     ``dim``, ``index``, ``eps``, ``activation`` ("gelu_tanh" unless given), ``name``; tensors ``<name>.gate | proj | norm``."""
+
+    reads_stream_input = True     # forward's ``h`` may be the residual itself in the run's dtype
 
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
@@ -126,8 +129,8 @@ class TokenSide(FeedForward):
         rows = batch.shared.get(SIDE_ROWS)
         if rows is None or rows.shape[1] < (self.index + 1) * self.dim:
             raise InvalidArgumentError("token_side: the embedding has left no side rows for this layer in the step")
-        x = residual
-        if self.runtime.dtype != torch.float32:
+        x = h if h is not None else residual
+        if h is None and self.runtime.dtype != torch.float32:
             x = self.runtime.empty((tokens, self.hidden))
             kernels.activation(residual, "none", x)
         gate = torch.empty((tokens, self.dim), dtype=torch.float32, device=residual.device)

@@ -80,7 +80,9 @@ class MixtureOfExperts(FeedForward):
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         self.w_router = tensors[base + "router"]
 
-    def forward(self, h, batch, residual, **_unused) -> None:
+    can_overwrite = True
+
+    def forward(self, h, batch, residual, accumulate: bool = True, **_unused) -> None:
         tokens = residual.shape[0]
         device = residual.device
         pairs = tokens * self.top
@@ -99,7 +101,7 @@ class MixtureOfExperts(FeedForward):
         act = self.runtime.empty((pairs, self.inter))
         pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
         kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,
-                            self.top, self.limit, self.alpha, act, pair_out, residual)
+                            self.top, self.limit, self.alpha, act, pair_out, residual, accumulate)
 
 
 register_ffn("moe", MixtureOfExperts)

@@ -44,9 +44,23 @@ class RMSNorm(Norm):
             weight = (weight.float() + 1.0).contiguous()
         self.weight = weight
 
-    def add_into(self, y: torch.Tensor, residual: torch.Tensor) -> None:
-        """``residual += y / rms(y) * gain``, all in 32-bit (the norm behind a sublayer)."""
+    def add_into(self, y: torch.Tensor, residual: torch.Tensor, follow=None, as_input: bool = False):
+        """``residual += y / rms(y) * gain``, all in 32-bit (the norm behind a sublayer).  ``follow``: the norm in front
+        of the next sublayer; if it is of this kind the same launch applies it to the new rows and its output is
+        returned.  ``as_input``: the new rows are returned in the run's dtype, for a part that reads the stream itself."""
+        if isinstance(follow, RMSNorm) and follow.weight is not None:
+            out = self.runtime.empty(tuple(residual.shape))
+            kernels.rmsnorm_add(y, self.weight, self.eps, residual, out, follow.weight, follow.eps)
+            return out
+        if as_input and follow is None:
+            if self.runtime.dtype == torch.float32:
+                kernels.rmsnorm_add(y, self.weight, self.eps, residual)
+                return residual
+            out = self.runtime.empty(tuple(residual.shape))
+            kernels.rmsnorm_add(y, self.weight, self.eps, residual, out)
+            return out
         kernels.rmsnorm_add(y, self.weight, self.eps, residual)
+        return follow.forward(residual) if follow is not None else None
 
     def handoff(self, tokens: int) -> Optional[NormHandoff]:
         if self.runtime.dtype != torch.bfloat16 or self.weight is None or self.weight.dtype != torch.float32:

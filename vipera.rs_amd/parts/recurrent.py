@@ -346,7 +346,12 @@ class SelectiveScan(Mixer):
         low = torch.empty((tokens, self.rank + 2 * self.states), **f32)
         linear(x32 if x_run is None else x_run, self.w_x, None, low)
         dt = torch.empty((tokens, self.inner), **f32)
-        linear(low[:, :self.rank], self.w_dt, None, dt)
+        steps = low[:, :self.rank]
+        if self.runtime.dtype != torch.float32 and self.w_dt.dtype == self.runtime.dtype and self.rank % 8 == 0:
+            # in the run's dtype the product runs on the matrix cores (a 32-bit input beside 16-bit weights would not)
+            steps = self.runtime.empty((tokens, self.rank))
+            kernels.activation(low[:, :self.rank], "none", steps)
+        linear(steps, self.w_dt, None, dt)
         y = self.runtime.empty((tokens, self.inner))
         z = xz[:, self.inner:]
         ahead = not batch.all_single
