@@ -408,6 +408,22 @@ def test_a_far_key_among_hundreds(tmp_path, mask, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dim, mask", [(64, 300), (128, 0)])
+def test_a_long_prompt_on_the_prompt_kernels_of_full_head_widths(tmp_path, dim, mask, dtype):
+    """Head widths of 64 and 128 take the prompt kernels that load tiles straight into LDS, which for a long prompt of
+    few heads cut a tile's positions into chunks or halves: blocks of 300 positions, capped scores and all positions
+    must come out of them as out of the others."""
+    cfg = Z.single(only_left(Z.left(4, 2, dim, dim, mask=mask, rot_dims=dim // 2, factor=4.0, softcap=10.0)), vocab=61, width=64)
+    folder = Z.make_folder(tmp_path / "long", cfg, 12)
+    cfg, w = Z.load_folder(folder)
+    tokens = Z.tokens_of(cfg["vocab"], 1300, 23)
+    want = P.forward(cfg, w, tokens)
+    runner = open_runner(folder, dtype, pages=90, page=16)
+    for plan in ([[(0, 1300)]], [[(0, 700)], [(0, 590)]] + [[(0, 1)]] * 10):
+        check(replay(runner, {0: tokens}, plan), {0: want}, TOL[dtype], "long prompt")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_slow_head_remembers_the_first_tokens(tmp_path, dtype):
     """A head that forgets nothing beside one that forgets at once: after 300 tokens, in pieces, the first tokens still
     weigh as much as the last, which a state that is lost or cleared between steps would not show."""

@@ -527,6 +527,45 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restric
   __shared__ float scratch[16];
   const float* src = y + (size_t)blockIdx.x * width;
   float* dst = residual + (size_t)blockIdx.x * width;
+  TO* out = next_out ? next_out + (size_t)blockIdx.x * width : nullptr;
+  constexpr int KEPT = 16;     // a row of up to 4,096 columns stays in registers: every operand is requested once, at the start
+  if (width <= KEPT * 256) {
+    float v[KEPT], x[KEPT], w[KEPT], nw[KEPT];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < KEPT; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      const bool in = c < width;
+      v[i] = in ? src[c] : 0.f;
+      x[i] = in ? dst[c] : 0.f;
+      w[i] = in ? weight[c] : 0.f;
+      nw[i] = (in && next_weight) ? next_weight[c] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < KEPT; ++i) sum += v[i] * v[i];
+    sum = block_sum(sum, scratch);
+    const float inv = 1.0f / sqrtf(sum / (float)width + eps);
+    float again = 0.f;
+#pragma unroll
+    for (int i = 0; i < KEPT; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      x[i] = x[i] + v[i] * inv * w[i];
+      if (c < width) dst[c] = x[i];
+      again += x[i] * x[i];
+    }
+    if (out == nullptr) return;
+    float next_inv = 1.0f;
+    if (next_weight) {
+      again = block_sum(again, scratch);
+      next_inv = 1.0f / sqrtf(again / (float)width + next_eps);
+    }
+#pragma unroll
+    for (int i = 0; i < KEPT; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (c < width) out[c] = from_float<TO>(next_weight ? x[i] * next_inv * nw[i] : x[i]);
+    }
+    return;
+  }
   float sum = 0.f;
   for (int i = threadIdx.x; i < width; i += 256) {
     const float v = src[i];
@@ -540,8 +579,7 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const float* __restric
     dst[i] = x;
     again += x * x;
   }
-  if (next_out == nullptr) return;
-  TO* out = next_out + (size_t)blockIdx.x * width;
+  if (out == nullptr) return;
   if (next_weight == nullptr) {
     for (int i = threadIdx.x; i < width; i += 256) out[i] = from_float<TO>(dst[i]);   // a thread reads what it wrote
     return;
