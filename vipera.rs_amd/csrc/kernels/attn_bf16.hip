@@ -156,7 +156,7 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 // State: o[DT] (O^T tiles), m (running max of the column), l (this lane's share of the running sum).
 // The loads of a step are issued one step ahead of its arithmetic (two operand sets that alternate by
 // unrolling): a wave has few steps and memory is the bound.
-template <bool REGS>
+template <bool REGS, bool EXT = true>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
                                              const CacheView& cv, float scale, float softcap, f32x4 (&o)[DT], float& m, float& l) {
   const int lane = threadIdx.x & 63, lg = lane >> 4;
@@ -186,7 +186,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
       for (int j = 0; j < 4; ++j) {
         const int p = kb + lg * 8 + sub * 4 + j;
         const bool visible = p >= col_lo && p <= col_pos && p >= begin && p < end;
-        const float x = visible ? capped(s[sub][j] * scale, softcap) : -INFINITY;
+        const float x = visible ? (EXT ? capped(s[sub][j] * scale, softcap) : s[sub][j] * scale) : -INFINITY;
         sv[sub * 4 + j] = x;
         tile_max = fmaxf(tile_max, x);
       }
@@ -897,7 +897,8 @@ constexpr int JOINED_WAVES = 8;
 #else
 #define VK_DECODE_WAVES_PER_SIMD 2
 #endif
-template <bool REGS, bool JOINED>
+// EXT: scores may be capped and `window` may be negative (blocks of positions); without it the kernel holds neither.
+template <bool REGS, bool JOINED, bool EXT>
 __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amdgpu_waves_per_eu(VK_DECODE_WAVES_PER_SIMD))) void attn_decode_kernel(
     const __bf16* __restrict__ q, long long q_stride, const __bf16* __restrict__ k_cache,
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, __bf16* __restrict__ out,
@@ -919,7 +920,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
   if (REGS && window == 0)
     early_pages = block_table[(size_t)entry * table_width + min(ps.page(chunk_index * chunk) + lane, table_width - 1)];
   const int pos = entry_first_pos[entry];
-  const int lo = first_visible(pos, window);
+  const int lo = EXT ? first_visible(pos, window) : ((window > 0 && pos + 1 > window) ? pos + 1 - window : 0);
   const int begin = max(lo, chunk_index * chunk), end = min(pos + 1, (chunk_index + 1) * chunk);
   const int head_in_group = hb * 16 + lr;
   const bool col_ok = head_in_group < group;
@@ -946,7 +947,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
       const int index = cv.page0 + lane;
       if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
     }
-    attend_range<REGS>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, softcap, o, m, l);
+    attend_range<REGS, EXT>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, softcap, o, m, l);
     l = sum_of_column(l);
   }
   if constexpr (JOINED) {
@@ -1180,17 +1181,20 @@ extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, con
   const int group = heads / kv_heads, head_blocks = (group + 15) / 16;
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
+  const bool ext = softcap > 0.f || window < 0;
   // pages a chunk can touch: chunks start at multiples of `chunk`, which need not be page edges
   const int chunk_pages = chunk % block_size == 0 ? chunk / block_size : chunk / block_size + 2;
   if (join) {
-    auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true, true> : attn_decode_kernel<false, true>;
+    auto kernel = ext ? (chunk_pages <= 64 ? attn_decode_kernel<true, true, true> : attn_decode_kernel<false, true, true>)
+                      : (chunk_pages <= 64 ? attn_decode_kernel<true, true, false> : attn_decode_kernel<false, true, false>);
     const int lds_bytes = chunks * (DT * 64 * 16 + 16 * 2 * 4);
-    static bool configured[2] = {false, false};
-    if (!configured[chunk_pages <= 64]) {
+    static bool configured[4] = {false, false, false, false};
+    const int which = (chunk_pages <= 64 ? 1 : 0) + (ext ? 2 : 0);
+    if (!configured[which]) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                          JOINED_WAVES * (DT * 64 * 16 + 16 * 2 * 4));
       if (e != hipSuccess) return (int)e;
-      configured[chunk_pages <= 64] = true;
+      configured[which] = true;
     }
     kernel<<<dim3(num_entries, kv_heads * head_blocks), chunks * 64, lds_bytes, s>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, nullptr, (__bf16*)out, entries,
@@ -1200,7 +1204,8 @@ extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, con
     return 0;
   }
   dim3 grid(num_entries, kv_heads * head_blocks, chunks);
-  auto kernel = chunk_pages <= 64 ? attn_decode_kernel<true, false> : attn_decode_kernel<false, false>;
+  auto kernel = ext ? (chunk_pages <= 64 ? attn_decode_kernel<true, false, true> : attn_decode_kernel<false, false, true>)
+                    : (chunk_pages <= 64 ? attn_decode_kernel<true, false, false> : attn_decode_kernel<false, false, false>);
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
                              (__bf16*)out, entries, entry_start, entry_first_pos, block_table, table_width, block_size,
                              heads, kv_heads, hd, scale, window, softcap, chunk, head_blocks, dense);
