@@ -8,10 +8,12 @@
 //
 // Both recurrences give the sixteen lanes of a quarter of a wave one output channel: each lane keeps R of the
 // channel's state numbers in registers, a sum over the state is R terms in a lane in ascending order and then four
-// exchanges inside the sixteen lanes.  That order depends on the sizes alone, so a token's result does not depend
-// on how its prompt was cut or on what else is in the step.  A workgroup (one wave) owns four channels of one entry and
-// walks the entry's tokens in order; the next token's operands are requested before the current one is worked on,
-// and no load sits behind a branch (a token past the entry's end reads the last one again).
+// DPP exchanges inside the sixteen lanes.  That order depends on the sizes alone, so a token's result does not depend
+// on how its prompt was cut or on what else is in the step.  A workgroup is one wave: four channels of one entry,
+// whose tokens it walks in order, a few tokens' operands on their way while the few before them are worked on; no
+// load sits behind a branch (a token past the entry's end reads the last one again).  What does not depend on the
+// state (activations of the inputs, the step sizes' softplus) is taken inside for steps of single tokens and once,
+// by a kernel ahead, for a prompt's portion, where every wave would pay for it token behind token.
 #include "common.h"
 
 __device__ __forceinline__ float scan_silu(float z) { return z / (1.0f + expf(-z)); }
